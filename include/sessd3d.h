@@ -57,7 +57,8 @@ enum {
     SESSD_E_NOMEM = 4
 };
 
-/* Bits of the device-side status word (last int32 of every workspace), read by *_status(). */
+/* Bits of the device-side status word (kept in the last 256-byte block of a layer's workspace and
+ * cleared by every enqueue), read back by *_status(). */
 enum {
     SESSD_STATUS_VOXEL_OVERFLOW = 1, /* more active sites than max_voxels; the excess was dropped  */
     SESSD_STATUS_HASH_FULL = 2,      /* hash table could not place a key (cannot happen when sized

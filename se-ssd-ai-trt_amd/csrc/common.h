@@ -1,0 +1,154 @@
+// common.h -- helpers shared by every translation unit of libsessd3d.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "../../include/sessd3d.h"
+
+namespace sessd {
+
+// ---------------------------------------------------------------------------------------------
+// error reporting: no abort(), a thread-local message and an error code instead
+// (the reference's checkCudaErrors prints and aborts, voxelGenerator.cu:8-19)
+// ---------------------------------------------------------------------------------------------
+void set_last_error(const std::string& msg);
+int fail(int code, const char* fmt, ...);
+
+#define SESSD_HIP_TRY(expr)                                                                      \
+    do {                                                                                         \
+        hipError_t e__ = (expr);                                                                 \
+        if (e__ != hipSuccess)                                                                   \
+            return ::sessd::fail(SESSD_E_HIP, "%s:%d: %s -> %s", __FILE__, __LINE__, #expr,      \
+                                 hipGetErrorString(e__));                                        \
+    } while (0)
+
+#define SESSD_TRY(expr)                  \
+    do {                                 \
+        int rc__ = (expr);               \
+        if (rc__ != SESSD_OK) return rc__; \
+    } while (0)
+
+// ---------------------------------------------------------------------------------------------
+// workspace carving: 256-byte aligned bump allocation, the same rule the reference uses
+// (alignPtr / nextWorkspacePtr / calculateTotalWorkspaceSize, submConv3dlayer.cu:93-124)
+// ---------------------------------------------------------------------------------------------
+constexpr size_t kWorkspaceAlign = 256;
+
+inline size_t align_up(size_t n, size_t a = kWorkspaceAlign) { return (n + a - 1) / a * a; }
+
+struct WorkspaceCarver {
+    uint8_t* base;
+    size_t offset = 0;
+    explicit WorkspaceCarver(void* p) : base(static_cast<uint8_t*>(p)) {}
+    template <typename T>
+    T* take(size_t count) {
+        T* p = base ? reinterpret_cast<T*>(base + offset) : nullptr;
+        offset += align_up(count * sizeof(T));
+        return p;
+    }
+    size_t total() const { return offset; }
+};
+
+inline uint32_t next_pow2(uint64_t v) {
+    uint32_t p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+inline int ilog2(uint32_t pow2) {
+    int l = 0;
+    while ((1u << l) < pow2) ++l;
+    return l;
+}
+inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+inline size_t dtype_size(int32_t t) { return t == SESSD_HALF ? 2 : 4; }
+
+constexpr uint32_t kEmpty = 0xFFFFFFFFu;
+
+// ---------------------------------------------------------------------------------------------
+// device side: open-addressing hash over linearised cell keys
+// ---------------------------------------------------------------------------------------------
+// keys[cap] (cap a power of two) start as kEmpty.  Multiplicative hashing spreads the strongly
+// correlated keys of neighbouring cells; linear probing keeps a probe sequence inside one or two
+// cache lines.  Every loop is bounded by the capacity: a full table is reported, never spun on.
+struct HashTable {
+    uint32_t* keys;
+    uint32_t* vals;
+    uint32_t mask;   // cap - 1
+    int32_t shift;   // 32 - log2(cap)
+};
+
+#ifdef __HIPCC__
+__device__ __forceinline__ uint32_t hash_slot0(const HashTable& t, uint32_t key) {
+    return (key * 2654435769u) >> t.shift;
+}
+
+// -> slot holding `key` (claimed now or earlier), or -1 when the table is full
+__device__ __forceinline__ int32_t hash_insert(const HashTable& t, uint32_t key) {
+    uint32_t slot = hash_slot0(t, key);
+    for (uint32_t probe = 0; probe <= t.mask; ++probe) {
+        uint32_t prev = atomicCAS(&t.keys[slot], kEmpty, key);
+        if (prev == kEmpty || prev == key) return (int32_t)slot;
+        slot = (slot + 1) & t.mask;
+    }
+    return -1;
+}
+
+// -> slot holding `key`, or -1 when absent
+__device__ __forceinline__ int32_t hash_find(const HashTable& t, uint32_t key) {
+    uint32_t slot = hash_slot0(t, key);
+    for (uint32_t probe = 0; probe <= t.mask; ++probe) {
+        uint32_t k = t.keys[slot];
+        if (k == key) return (int32_t)slot;
+        if (k == kEmpty) return -1;
+        slot = (slot + 1) & t.mask;
+    }
+    return -1;
+}
+
+__device__ __forceinline__ uint32_t lane_id() { return __lane_id(); }
+
+// number of set bits of `m` below this lane (wave64)
+__device__ __forceinline__ uint32_t rank_in_wave(uint64_t m) {
+    return __popcll(m & ((1ull << lane_id()) - 1ull));
+}
+#endif
+
+inline HashTable make_hash(uint32_t* keys, uint32_t* vals, uint32_t cap) {
+    HashTable t;
+    t.keys = keys;
+    t.vals = vals;
+    t.mask = cap - 1;
+    t.shift = 32 - ilog2(cap);
+    return t;
+}
+
+// ---------------------------------------------------------------------------------------------
+// fill: the only way memory is cleared (a kernel, so an enqueue can be captured in a hipGraph)
+// ---------------------------------------------------------------------------------------------
+struct FillRegion {
+    uint32_t* ptr;     // 16-byte aligned
+    uint64_t words;    // 32-bit words
+    uint32_t value;
+};
+struct FillArgs {
+    FillRegion r[6];
+    int n = 0;
+    void add(void* p, uint64_t words, uint32_t value) {
+        if (!p || !words) return;
+        r[n].ptr = static_cast<uint32_t*>(p);
+        r[n].words = words;
+        r[n].value = value;
+        ++n;
+    }
+};
+int launch_fill(const FillArgs& a, hipStream_t stream);
+
+}  // namespace sessd

@@ -1,0 +1,39 @@
+// kernels.h -- launchers of the gather-GEMM kernels (conv_gemm.hip) used by both conv plugins.
+#pragma once
+
+#include "common.h"
+
+namespace sessd {
+
+struct GemmArgs {
+    const void* in_feat;     // [max_voxels][cin]   FP32 or FP16
+    void* out_feat;          // [max_voxels][cout]  FP32 or FP16
+    const int32_t* nbr;      // [K][max_voxels] input row feeding (offset k, output row), -1 = none
+    const int32_t* num_out;  // device scalar: active output rows
+    int max_voxels;
+    int K, cin, cout;
+    int in_type, out_type;   // SESSD_FLOAT / SESSD_HALF
+    const float* w_f32;      // [K][cin][cout]
+    const __half* w_f16;     // same layout, rounded to half (used when in_type is HALF)
+    const void* w_packed;    // MFMA operand order, or null
+    const float* scale;      // [cout] or null
+    const float* shift;      // [cout] or null
+    int relu;
+    int write_pad_rows;      // rows >= *num_out get epilogue(0) (the reference zero-fills them)
+};
+
+// picks the kernel for the layer shape; returns SESSD_E_UNSUPPORTED for dtype pairs not covered
+int launch_gather_gemm(const GemmArgs& a, hipStream_t stream);
+
+// size in bytes of the packed weight copy for this shape/dtype (0 = shape runs on the VALU path)
+size_t packed_weight_bytes(int K, int cin, int cout, int dtype);
+// host-side packing into MFMA operand order; dst has packed_weight_bytes() bytes
+void pack_weights(const float* w, int K, int cin, int cout, int dtype, void* dst);
+
+// rulebook export (reference layout indice_pairs[K][2][max_voxels], indice_num[K])
+size_t export_scratch_bytes(int K, int max_voxels);
+int launch_export_rulebook(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels,
+                           void* scratch, int32_t* indice_pairs, uint32_t* indice_num,
+                           hipStream_t stream);
+
+}  // namespace sessd

@@ -1,0 +1,381 @@
+// pipeline.hip -- frame pipeline: VoxelGenerator -> conv stack -> Sparse2Dense on one stream.
+//
+// Counterpart of the graph the reference wires in createEngine (se-ssd-ai-trt.cpp:1138-1252) and of
+// what TensorRT's executor does at run time: it owns every intermediate tensor and workspace and
+// calls each plugin's enqueue in order.  BatchNorm1d + ReLU (se-ssd-ai-trt.cpp:808-856) is folded
+// into each conv's epilogue.  Everything is allocated in create(); enqueue only launches kernels,
+// optionally by replaying a hipGraph captured from the same enqueue sequence.
+#include <memory>
+
+#include "plugins.h"
+
+namespace sessd {
+
+namespace {
+
+sessd_tensor_desc make_desc(std::initializer_list<int> dims, int type) {
+    sessd_tensor_desc t;
+    std::memset(&t, 0, sizeof(t));
+    t.nbDims = (int)dims.size();
+    int i = 0;
+    for (int v : dims) t.d[i++] = v;
+    t.type = type;
+    t.scale = 1.0f;
+    return t;
+}
+
+struct DeviceBuffer {
+    void* p = nullptr;
+    size_t bytes = 0;
+    int alloc(size_t n) {
+        bytes = n;
+        SESSD_HIP_TRY(hipMalloc(&p, n ? n : 16));
+        return SESSD_OK;
+    }
+    ~DeviceBuffer() {
+        if (p) (void)hipFree(p);
+    }
+};
+
+}  // namespace
+
+struct ConvStage {
+    sessd_layer_spec spec;
+    std::unique_ptr<SubmConv3dLayerPlugin> subm;
+    std::unique_ptr<SparseConv3dLayerPlugin> sparse;
+    DeviceBuffer ws, feat, coors, num;  // coors/num only for sparse layers (they produce new ones)
+    int rulebook_from = -1;             // SubM layer whose workspace holds this layer's rulebook
+    sessd_tensor_desc in_desc[3], out_desc[3];
+    void* coors_ptr = nullptr;  // coordinates valid AFTER this layer
+    void* num_ptr = nullptr;
+};
+
+struct Pipeline {
+    sessd_pipeline_desc desc;
+    std::unique_ptr<VoxelGeneratorPlugin> vg;
+    std::unique_ptr<Sparse2DensePlugin> s2d;
+    std::vector<std::unique_ptr<ConvStage>> stages;
+    DeviceBuffer vg_ws, vg_voxels, vg_coors, vg_num, s2d_ws;
+    sessd_tensor_desc vg_in[2], vg_out[3], s2d_in[3], s2d_out[1];
+    int max_voxels = 0;
+    size_t device_bytes = 0;
+    // graph replay
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    const void* g_points = nullptr;
+    const void* g_size = nullptr;
+    void* g_dense = nullptr;
+    int graph_nodes = -1;
+
+    ~Pipeline() {
+        if (graph_exec) (void)hipGraphExecDestroy(graph_exec);
+        if (graph) (void)hipGraphDestroy(graph);
+    }
+
+    int enqueueDirect(const void* points, const void* points_size, void* dense, hipStream_t stream) {
+        const void* vin[2] = {points, points_size};
+        void* vout[3] = {vg_voxels.p, vg_coors.p, vg_num.p};
+        SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, stream));
+        const void* feat = vg_voxels.p;
+        const void* coors = vg_coors.p;
+        const void* num = vg_num.p;
+        for (auto& st : stages) {
+            const void* in[3] = {feat, coors, num};
+            if (st->subm) {
+                void* out[1] = {st->feat.p};
+                if (st->rulebook_from >= 0)
+                    SESSD_TRY(st->subm->enqueueShared(st->in_desc, st->out_desc, in, out,
+                                                      stages[st->rulebook_from]->ws.p, stream));
+                else
+                    SESSD_TRY(st->subm->enqueue(st->in_desc, st->out_desc, in, out, st->ws.p, stream));
+            } else {
+                void* out[3] = {st->feat.p, st->coors.p, st->num.p};
+                SESSD_TRY(st->sparse->enqueue(st->in_desc, st->out_desc, in, out, st->ws.p, stream));
+                coors = st->coors.p;
+                num = st->num.p;
+            }
+            feat = st->feat.p;
+        }
+        const void* din[3] = {feat, coors, num};
+        void* dout[1] = {dense};
+        return s2d->enqueue(s2d_in, s2d_out, din, dout, s2d_ws.p, stream);
+    }
+};
+
+static int build_pipeline(const sessd_pipeline_desc& d, Pipeline* P) {
+    if (d.n_layers < 0 || (d.n_layers && (!d.layers || !d.weights)))
+        return fail(SESSD_E_INVALID, "pipeline: layers/weights missing");
+    if (d.feature_dtype != SESSD_FLOAT && d.feature_dtype != SESSD_HALF)
+        return fail(SESSD_E_UNSUPPORTED, "pipeline: feature_dtype must be FP32 or FP16");
+    if (d.max_points <= 0 || d.point_features < 4) return fail(SESSD_E_INVALID, "pipeline: bad points shape");
+    P->desc = d;
+    const int V = d.voxelgen.max_voxels;
+    P->max_voxels = V;
+    const int ft = d.feature_dtype;
+    size_t total = 0;
+
+    VoxelGeneratorPlugin* vg = nullptr;
+    SESSD_TRY(VoxelGeneratorPlugin::create(d.voxelgen, &vg));
+    P->vg.reset(vg);
+    vg->flags_ = d.flags;
+    P->vg_in[0] = make_desc({1, d.max_points, d.point_features}, SESSD_FLOAT);
+    P->vg_in[1] = make_desc({1}, SESSD_INT32);
+    P->vg_out[0] = make_desc({1, V, 4}, SESSD_FLOAT);
+    P->vg_out[1] = make_desc({1, V, 4}, SESSD_INT32);
+    P->vg_out[2] = make_desc({1}, SESSD_INT32);
+    SESSD_TRY(vg->configurePlugin(P->vg_in, 2, P->vg_out, 3));
+    SESSD_TRY(P->vg_ws.alloc(vg->getWorkspaceSize(P->vg_in, 2, P->vg_out, 3)));
+    SESSD_TRY(P->vg_voxels.alloc((size_t)V * 4 * sizeof(float)));
+    SESSD_TRY(P->vg_coors.alloc((size_t)V * 4 * sizeof(int32_t)));
+    SESSD_TRY(P->vg_num.alloc(256));
+    total += P->vg_ws.bytes + P->vg_voxels.bytes + P->vg_coors.bytes + 256;
+
+    int in_type = SESSD_FLOAT;  // the voxelizer's means are FP32
+    int in_ch = 4;
+    int last_subm_with_rulebook = -1;
+    for (int l = 0; l < d.n_layers; ++l) {
+        const sessd_layer_spec& s = d.layers[l];
+        if (s.in_channel != in_ch)
+            return fail(SESSD_E_INVALID, "pipeline: layer %d expects %d input channels, previous layer has %d", l,
+                        s.in_channel, in_ch);
+        auto st = std::make_unique<ConvStage>();
+        st->spec = s;
+        st->in_desc[0] = make_desc({1, V, s.in_channel}, in_type);
+        st->in_desc[1] = make_desc({1, V, 4}, SESSD_INT32);
+        st->in_desc[2] = make_desc({1}, SESSD_INT32);
+        st->out_desc[0] = make_desc({1, V, s.out_channel}, ft);
+        st->out_desc[1] = make_desc({1, V, 4}, SESSD_INT32);
+        st->out_desc[2] = make_desc({1}, SESSD_INT32);
+        ConvPluginBase* base = nullptr;
+        if (s.type == SESSD_LAYER_SUBM) {
+            sessd_submconv3d_desc cd;
+            std::memset(&cd, 0, sizeof(cd));
+            cd.in_channel = s.in_channel;
+            cd.out_channel = s.out_channel;
+            cd.max_voxels = V;
+            cd.feature_num = s.in_channel;  // se-ssd-ai-trt.cpp:739
+            for (int a = 0; a < 3; ++a) cd.out_shape[a] = cd.spatial_shape[a] = s.out_shape[a];
+            cd.ksize = s.ksize[0];
+            cd.stride = s.stride[0];
+            cd.padding = s.padding[0];
+            cd.dilation = 1;
+            SubmConv3dLayerPlugin* p = nullptr;
+            SESSD_TRY(SubmConv3dLayerPlugin::create(cd, d.weights[l], &p));
+            st->subm.reset(p);
+            base = p;
+            SESSD_TRY(p->configurePlugin(st->in_desc, 3, st->out_desc, 1));
+            if (d.share_rulebooks && last_subm_with_rulebook >= 0) {
+                const sessd_layer_spec& o = d.layers[last_subm_with_rulebook];
+                bool same = o.ksize[0] == s.ksize[0] && o.padding[0] == s.padding[0];
+                for (int a = 0; a < 3; ++a) same = same && o.out_shape[a] == s.out_shape[a];
+                if (same) st->rulebook_from = last_subm_with_rulebook;
+            }
+            if (st->rulebook_from < 0) {
+                SESSD_TRY(st->ws.alloc(p->getWorkspaceSize(st->in_desc, 3, st->out_desc, 1)));
+                last_subm_with_rulebook = l;
+            }
+        } else if (s.type == SESSD_LAYER_SPARSE) {
+            sessd_sparseconv3d_desc cd;
+            std::memset(&cd, 0, sizeof(cd));
+            cd.in_channel = s.in_channel;
+            cd.out_channel = s.out_channel;
+            cd.max_voxels = V;
+            cd.feature_num = s.in_channel;
+            for (int a = 0; a < 3; ++a) {
+                cd.out_shape[a] = s.out_shape[a];
+                cd.ksize[a] = s.ksize[a];
+                cd.stride[a] = s.stride[a];
+                cd.padding[a] = s.padding[a];
+            }
+            cd.dilation = 1;
+            SparseConv3dLayerPlugin* p = nullptr;
+            SESSD_TRY(SparseConv3dLayerPlugin::create(cd, d.weights[l], &p));
+            st->sparse.reset(p);
+            base = p;
+            SESSD_TRY(p->configurePlugin(st->in_desc, 3, st->out_desc, 3));
+            SESSD_TRY(st->ws.alloc(p->getWorkspaceSize(st->in_desc, 3, st->out_desc, 3)));
+            SESSD_TRY(st->coors.alloc((size_t)V * 4 * sizeof(int32_t)));
+            SESSD_TRY(st->num.alloc(256));
+            last_subm_with_rulebook = -1;  // new coordinates: earlier rulebooks no longer apply
+        } else {
+            return fail(SESSD_E_INVALID, "pipeline: layer %d has unknown type %d", l, s.type);
+        }
+        base->flags_ = d.flags;
+        SESSD_TRY(base->setEpilogue(d.scale ? d.scale[l] : nullptr, d.shift ? d.shift[l] : nullptr, d.relu));
+        SESSD_TRY(st->feat.alloc((size_t)V * s.out_channel * dtype_size(ft)));
+        total += st->ws.bytes + st->feat.bytes + st->coors.bytes + st->num.bytes;
+        in_type = ft;
+        in_ch = s.out_channel;
+        P->stages.push_back(std::move(st));
+    }
+
+    if (d.dense.feature_map_channel != in_ch)
+        return fail(SESSD_E_INVALID, "pipeline: sparse2dense expects %d channels, backbone ends with %d",
+                    d.dense.feature_map_channel, in_ch);
+    Sparse2DensePlugin* s2d = nullptr;
+    SESSD_TRY(Sparse2DensePlugin::create(d.dense, &s2d));
+    P->s2d.reset(s2d);
+    P->s2d_in[0] = make_desc({1, V, in_ch}, in_type);
+    P->s2d_in[1] = make_desc({1, V, 4}, SESSD_INT32);
+    P->s2d_in[2] = make_desc({1}, SESSD_INT32);
+    P->s2d_out[0] = make_desc({1, d.dense.feature_map_channel * d.dense.feature_map_size[2],
+                               d.dense.feature_map_size[1], d.dense.feature_map_size[0]}, ft);
+    SESSD_TRY(s2d->configurePlugin(P->s2d_in, 3, P->s2d_out, 1));
+    SESSD_TRY(P->s2d_ws.alloc(s2d->getWorkspaceSize(P->s2d_in, 3, P->s2d_out, 1)));
+    total += P->s2d_ws.bytes;
+    P->device_bytes = total;
+    // the layer array of the caller need not outlive create()
+    P->desc.layers = nullptr;
+    P->desc.weights = P->desc.scale = P->desc.shift = nullptr;
+    return SESSD_OK;
+}
+
+}  // namespace sessd
+
+using namespace sessd;
+
+extern "C" {
+
+int sessd_reference_backbone(sessd_layer_spec* layers, int max_layers, sessd_voxelgen_desc* voxelgen,
+                             sessd_sparse2dense_desc* dense) {
+    // params.h:39-192: {type, cin, cout, ksize zyx, stride zyx, padding zyx, out_shape xyz}
+    static const sessd_layer_spec table[14] = {
+        {SESSD_LAYER_SUBM, 4, 16, {3, 3, 3}, {1, 1, 1}, {1, 1, 1}, {1408, 1600, 41}},
+        {SESSD_LAYER_SUBM, 16, 16, {3, 3, 3}, {1, 1, 1}, {1, 1, 1}, {1408, 1600, 41}},
+        {SESSD_LAYER_SPARSE, 16, 32, {3, 3, 3}, {2, 2, 2}, {1, 1, 1}, {704, 800, 21}},
+        {SESSD_LAYER_SUBM, 32, 32, {3, 3, 3}, {1, 1, 1}, {1, 1, 1}, {704, 800, 21}},
+        {SESSD_LAYER_SUBM, 32, 32, {3, 3, 3}, {1, 1, 1}, {1, 1, 1}, {704, 800, 21}},
+        {SESSD_LAYER_SPARSE, 32, 64, {3, 3, 3}, {2, 2, 2}, {1, 1, 1}, {352, 400, 11}},
+        {SESSD_LAYER_SUBM, 64, 64, {3, 3, 3}, {1, 1, 1}, {1, 1, 1}, {352, 400, 11}},
+        {SESSD_LAYER_SUBM, 64, 64, {3, 3, 3}, {1, 1, 1}, {1, 1, 1}, {352, 400, 11}},
+        {SESSD_LAYER_SUBM, 64, 64, {3, 3, 3}, {1, 1, 1}, {1, 1, 1}, {352, 400, 11}},
+        {SESSD_LAYER_SPARSE, 64, 64, {3, 3, 3}, {2, 2, 2}, {0, 1, 1}, {176, 200, 5}},
+        {SESSD_LAYER_SUBM, 64, 64, {3, 3, 3}, {1, 1, 1}, {1, 1, 1}, {176, 200, 5}},
+        {SESSD_LAYER_SUBM, 64, 64, {3, 3, 3}, {1, 1, 1}, {1, 1, 1}, {176, 200, 5}},
+        {SESSD_LAYER_SUBM, 64, 64, {3, 3, 3}, {1, 1, 1}, {1, 1, 1}, {176, 200, 5}},
+        {SESSD_LAYER_SPARSE, 64, 64, {3, 1, 1}, {2, 1, 1}, {0, 0, 0}, {176, 200, 2}},
+    };
+    int n = 0;
+    if (layers)
+        for (; n < 14 && n < max_layers; ++n) layers[n] = table[n];
+    if (voxelgen) {  // params.h:19-36
+        voxelgen->max_num_points_per_voxel = 5;
+        voxelgen->max_voxels = 60000;
+        const float r[6] = {0.0f, -40.0f, -3.0f, 70.4f, 40.0f, 1.0f};
+        for (int i = 0; i < 6; ++i) voxelgen->point_cloud_range[i] = r[i];
+        voxelgen->voxel_feature_num = 4;
+        voxelgen->voxel_size[0] = 0.05f;
+        voxelgen->voxel_size[1] = 0.05f;
+        voxelgen->voxel_size[2] = 0.1f;
+    }
+    if (dense) {  // params.h:194-197
+        dense->feature_map_size[0] = 176;
+        dense->feature_map_size[1] = 200;
+        dense->feature_map_size[2] = 2;
+        dense->feature_map_channel = 64;
+    }
+    return n;
+}
+
+int sessd_pipeline_create(const sessd_pipeline_desc* desc, sessd_pipeline** out) {
+    if (!desc || !out) return fail(SESSD_E_INVALID, "pipeline_create: null argument");
+    auto* P = new Pipeline();
+    const int rc = build_pipeline(*desc, P);
+    if (rc != SESSD_OK) {
+        delete P;
+        return rc;
+    }
+    *out = reinterpret_cast<sessd_pipeline*>(P);
+    return SESSD_OK;
+}
+
+int sessd_pipeline_enqueue(sessd_pipeline* h, const void* points, const void* points_size, void* dense,
+                           sessd_stream_t stream_) {
+    if (!h || !points || !points_size || !dense) return fail(SESSD_E_INVALID, "pipeline_enqueue: null argument");
+    auto* P = reinterpret_cast<Pipeline*>(h);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (!P->desc.use_graph || stream == nullptr) return P->enqueueDirect(points, points_size, dense, stream);
+    if (!P->graph_exec || P->g_points != points || P->g_size != points_size || P->g_dense != dense) {
+        if (P->graph_exec) (void)hipGraphExecDestroy(P->graph_exec);
+        if (P->graph) (void)hipGraphDestroy(P->graph);
+        P->graph_exec = nullptr;
+        P->graph = nullptr;
+        SESSD_HIP_TRY(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+        const int rc = P->enqueueDirect(points, points_size, dense, stream);
+        hipGraph_t g = nullptr;
+        const hipError_t e = hipStreamEndCapture(stream, &g);
+        if (rc != SESSD_OK) {
+            if (g) (void)hipGraphDestroy(g);
+            return rc;
+        }
+        if (e != hipSuccess) return fail(SESSD_E_HIP, "pipeline: stream capture failed: %s", hipGetErrorString(e));
+        P->graph = g;
+        SESSD_HIP_TRY(hipGraphInstantiate(&P->graph_exec, P->graph, nullptr, nullptr, 0));
+        size_t nodes = 0;
+        if (hipGraphGetNodes(P->graph, nullptr, &nodes) == hipSuccess) P->graph_nodes = (int)nodes;
+        P->g_points = points;
+        P->g_size = points_size;
+        P->g_dense = dense;
+    }
+    SESSD_HIP_TRY(hipGraphLaunch(P->graph_exec, stream));
+    return SESSD_OK;
+}
+
+int sessd_pipeline_layer_io(sessd_pipeline* h, int layer, void** feat, void** coors, void** voxel_num,
+                            void** workspace, int32_t* channels) {
+    if (!h) return fail(SESSD_E_INVALID, "pipeline_layer_io: null handle");
+    auto* P = reinterpret_cast<Pipeline*>(h);
+    if (layer < -1 || layer >= (int)P->stages.size()) return fail(SESSD_E_INVALID, "pipeline_layer_io: no layer %d", layer);
+    void* f = P->vg_voxels.p;
+    void* c = P->vg_coors.p;
+    void* n = P->vg_num.p;
+    void* w = P->vg_ws.p;
+    int ch = 4;
+    for (int l = 0; l <= layer; ++l) {
+        ConvStage& st = *P->stages[l];
+        f = st.feat.p;
+        ch = st.spec.out_channel;
+        if (st.sparse) {
+            c = st.coors.p;
+            n = st.num.p;
+        }
+        w = st.rulebook_from >= 0 ? P->stages[st.rulebook_from]->ws.p : st.ws.p;
+    }
+    if (feat) *feat = f;
+    if (coors) *coors = c;
+    if (voxel_num) *voxel_num = n;
+    if (workspace) *workspace = w;
+    if (channels) *channels = ch;
+    return SESSD_OK;
+}
+
+int sessd_pipeline_status(sessd_pipeline* h, sessd_stream_t stream_, int32_t* status) {
+    if (!h || !status) return fail(SESSD_E_INVALID, "pipeline_status: null argument");
+    auto* P = reinterpret_cast<Pipeline*>(h);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    int32_t acc = 0, s = 0;
+    SESSD_TRY(read_status_word(P->vg_ws.p, P->vg->statusOffset(P->desc.max_points), stream, &s));
+    acc |= s;
+    for (auto& st : P->stages) {
+        if (!st->ws.p) continue;
+        const size_t off = st->subm ? st->subm->statusOffset() : st->sparse->statusOffset();
+        SESSD_TRY(read_status_word(st->ws.p, off, stream, &s));
+        acc |= s;
+    }
+    SESSD_TRY(read_status_word(P->s2d_ws.p, 0, stream, &s));
+    acc |= s;
+    *status = acc;
+    return SESSD_OK;
+}
+
+size_t sessd_pipeline_device_bytes(const sessd_pipeline* h) {
+    return h ? reinterpret_cast<const Pipeline*>(h)->device_bytes : 0;
+}
+
+int sessd_pipeline_num_launches(const sessd_pipeline* h) {
+    return h ? reinterpret_cast<const Pipeline*>(h)->graph_nodes : -1;
+}
+
+void sessd_pipeline_destroy(sessd_pipeline* h) { delete reinterpret_cast<Pipeline*>(h); }
+
+}  // extern "C"

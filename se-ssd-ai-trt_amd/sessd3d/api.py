@@ -1,0 +1,437 @@
+"""ctypes binding of libsessd3d.so plus thin per-plugin wrappers.
+
+torch is used only to own device memory and streams; every compute call goes through the C-ABI
+declared in include/sessd3d.h.  There is no fallback: if the library is missing the import of
+`lib()` raises.
+"""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+
+from . import backbone as B
+from . import ctypes_defs as D
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libsessd3d.so")
+HEADER_PATH = os.path.join(os.path.dirname(os.path.dirname(_HERE)), "include", "sessd3d.h")
+_lib = None
+
+
+class SessdError(RuntimeError):
+    pass
+
+
+def declared_symbols():
+    """Names of all functions declared in include/sessd3d.h."""
+    with open(HEADER_PATH) as f:
+        text = f.read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sessd_[a-z0-9_]+)\s*\(", text)))
+
+
+def lib():
+    """Load libsessd3d.so (built by se-ssd-ai-trt_amd/build.py).  Never falls back to anything else."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise SessdError("libsessd3d.so is not built: run `python se-ssd-ai-trt_amd/build.py` (%s)" % LIB_PATH)
+    L = C.CDLL(LIB_PATH)
+    vp, sz, i32 = C.c_void_p, C.c_size_t, C.c_int32
+    TD = C.POINTER(D.TensorDesc)
+    VPP = C.POINTER(C.c_void_p)
+    L.sessd_last_error.restype = C.c_char_p
+    L.sessd_version.restype = C.c_char_p
+    for name in ("voxelgen", "submconv3d", "sparseconv3d", "sparse2dense"):
+        getattr(L, "sessd_%s_serialization_size" % name).restype = sz
+        getattr(L, "sessd_%s_serialization_size" % name).argtypes = [vp]
+        getattr(L, "sessd_%s_serialize" % name).argtypes = [vp, vp]
+        getattr(L, "sessd_%s_deserialize" % name).argtypes = [vp, sz, VPP]
+        getattr(L, "sessd_%s_configure" % name).argtypes = [vp, TD, C.c_int, TD, C.c_int]
+        getattr(L, "sessd_%s_workspace_size" % name).restype = sz
+        getattr(L, "sessd_%s_workspace_size" % name).argtypes = [vp, TD, C.c_int, TD, C.c_int]
+        getattr(L, "sessd_%s_enqueue" % name).argtypes = [vp, TD, TD, VPP, VPP, vp, vp]
+        getattr(L, "sessd_%s_destroy" % name).argtypes = [vp]
+        getattr(L, "sessd_%s_destroy" % name).restype = None
+    for name in ("voxelgen", "submconv3d", "sparseconv3d"):
+        getattr(L, "sessd_%s_status" % name).argtypes = [vp, vp, vp, C.POINTER(i32)]
+        getattr(L, "sessd_%s_set_flags" % name).argtypes = [vp, i32]
+    for name in ("submconv3d", "sparseconv3d"):
+        getattr(L, "sessd_%s_set_epilogue" % name).argtypes = [vp, vp, vp, C.c_int]
+        getattr(L, "sessd_%s_export_rulebook" % name).argtypes = [vp, vp, vp, vp, vp]
+    L.sessd_voxelgen_create.argtypes = [C.POINTER(D.VoxelGenDesc), VPP]
+    L.sessd_voxelgen_grid_size.argtypes = [vp, C.POINTER(i32)]
+    L.sessd_submconv3d_create.argtypes = [C.POINTER(D.SubmConv3dDesc), vp, VPP]
+    L.sessd_submconv3d_enqueue_shared.argtypes = [vp, TD, TD, VPP, VPP, vp, vp]
+    L.sessd_sparseconv3d_create.argtypes = [C.POINTER(D.SparseConv3dDesc), vp, VPP]
+    L.sessd_sparse2dense_create.argtypes = [C.POINTER(D.Sparse2DenseDesc), VPP]
+    L.sessd_reference_backbone.argtypes = [C.POINTER(D.LayerSpec), C.c_int, C.POINTER(D.VoxelGenDesc),
+                                           C.POINTER(D.Sparse2DenseDesc)]
+    L.sessd_pipeline_create.argtypes = [C.POINTER(D.PipelineDesc), VPP]
+    L.sessd_pipeline_enqueue.argtypes = [vp, vp, vp, vp, vp]
+    L.sessd_pipeline_layer_io.argtypes = [vp, C.c_int, VPP, VPP, VPP, VPP, C.POINTER(i32)]
+    L.sessd_pipeline_status.argtypes = [vp, vp, C.POINTER(i32)]
+    L.sessd_pipeline_device_bytes.restype = sz
+    L.sessd_pipeline_device_bytes.argtypes = [vp]
+    L.sessd_pipeline_num_launches.argtypes = [vp]
+    L.sessd_pipeline_destroy.argtypes = [vp]
+    L.sessd_pipeline_destroy.restype = None
+    _lib = L
+    return L
+
+
+def check(rc):
+    if rc != 0:
+        raise SessdError("sessd3d error %d: %s" % (rc, lib().sessd_last_error().decode()))
+
+
+def _torch():
+    import torch
+    return torch
+
+
+def _stream_ptr(stream=None):
+    torch = _torch()
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return C.c_void_p(s.cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _np_f32_ptr(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else C.c_void_p(0)
+
+
+def _dtype_code(t):
+    torch = _torch()
+    return {torch.float32: D.SESSD_FLOAT, torch.float16: D.SESSD_HALF, torch.int32: D.SESSD_INT32}[t.dtype]
+
+
+def _descs(tensors):
+    arr = (D.TensorDesc * len(tensors))()
+    for i, t in enumerate(tensors):
+        dims = [1] + list(t.shape) if t.dim() >= 2 else list(t.shape)
+        arr[i] = D.TensorDesc.make(dims, _dtype_code(t))
+    return arr
+
+
+def _voidpp(tensors):
+    return (C.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+class _Plugin:
+    """Life cycle shared by the four plugin wrappers; `kind` is the symbol infix."""
+    kind = ""
+
+    def __init__(self, handle):
+        self.h = handle
+        self.ws = None
+
+    def _fn(self, name):
+        return getattr(lib(), "sessd_%s_%s" % (self.kind, name))
+
+    def serialize(self) -> bytes:
+        n = self._fn("serialization_size")(self.h)
+        buf = C.create_string_buffer(n)
+        check(self._fn("serialize")(self.h, buf))
+        return buf.raw
+
+    @classmethod
+    def deserialize(cls, blob: bytes):
+        h = C.c_void_p()
+        check(getattr(lib(), "sessd_%s_deserialize" % cls.kind)(blob, len(blob), C.byref(h)))
+        obj = cls.__new__(cls)
+        _Plugin.__init__(obj, h)
+        return obj
+
+    def configure(self, inputs, outputs):
+        check(self._fn("configure")(self.h, _descs(inputs), len(inputs), _descs(outputs), len(outputs)))
+
+    def workspace_size(self, inputs, outputs) -> int:
+        return self._fn("workspace_size")(self.h, _descs(inputs), len(inputs), _descs(outputs), len(outputs))
+
+    def _workspace(self, inputs, outputs):
+        torch = _torch()
+        n = self.workspace_size(inputs, outputs)
+        if self.ws is None or self.ws.numel() < n:
+            self.ws = torch.empty(max(n, 256), dtype=torch.uint8, device=inputs[0].device)
+        return self.ws
+
+    def enqueue(self, inputs, outputs, stream=None, workspace=None):
+        """inputs/outputs: lists of torch device tensors without the batch dimension."""
+        ws = workspace if workspace is not None else self._workspace(inputs, outputs)
+        check(self._fn("enqueue")(self.h, _descs(inputs), _descs(outputs), _voidpp(inputs), _voidpp(outputs),
+                                  _ptr(ws), _stream_ptr(stream)))
+        return ws
+
+    def status(self, stream=None) -> int:
+        s = C.c_int32(0)
+        check(self._fn("status")(self.h, _ptr(self.ws), _stream_ptr(stream), C.byref(s)))
+        return s.value
+
+    def set_flags(self, flags):
+        check(self._fn("set_flags")(self.h, flags))
+
+    def close(self):
+        if self.h:
+            self._fn("destroy")(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class VoxelGenerator(_Plugin):
+    kind = "voxelgen"
+
+    def __init__(self, max_voxels=B.MAX_VOXELS, max_num_points_per_voxel=B.MAX_NUM_POINTS_PER_VOXEL,
+                 point_cloud_range=B.POINT_CLOUD_RANGE, voxel_size=B.VOXEL_SIZE):
+        d = B.voxelgen_desc(max_voxels, max_num_points_per_voxel, point_cloud_range, voxel_size)
+        h = C.c_void_p()
+        check(lib().sessd_voxelgen_create(C.byref(d), C.byref(h)))
+        super().__init__(h)
+        self.max_voxels = max_voxels
+
+    def grid_size(self):
+        g = (C.c_int32 * 3)()
+        check(lib().sessd_voxelgen_grid_size(self.h, g))
+        return tuple(g)
+
+    def __call__(self, points, points_size, stream=None):
+        """points f32[max_points,F], points_size i32[1] (device) -> voxels, coors, voxel_num (device)"""
+        torch = _torch()
+        dev = points.device
+        voxels = torch.empty((self.max_voxels, 4), dtype=torch.float32, device=dev)
+        coors = torch.empty((self.max_voxels, 4), dtype=torch.int32, device=dev)
+        num = torch.empty((1,), dtype=torch.int32, device=dev)
+        self.configure([points, points_size], [voxels, coors, num])
+        self.enqueue([points, points_size], [voxels, coors, num], stream)
+        return voxels, coors, num
+
+
+class _Conv(_Plugin):
+    def set_epilogue(self, scale=None, shift=None, relu=True):
+        sc = None if scale is None else np.ascontiguousarray(scale, np.float32)
+        sh = None if shift is None else np.ascontiguousarray(shift, np.float32)
+        check(self._fn("set_epilogue")(self.h, _np_f32_ptr(sc), _np_f32_ptr(sh), int(relu)))
+
+    def export_rulebook(self, stream=None, workspace=None):
+        """-> indice_pairs i32[K,2,max_voxels], indice_num i32[K] (device tensors)"""
+        torch = _torch()
+        ws = workspace if workspace is not None else self.ws
+        pairs = torch.empty((self.kvol, 2, self.max_voxels), dtype=torch.int32, device=ws.device)
+        num = torch.empty((self.kvol,), dtype=torch.int32, device=ws.device)
+        check(self._fn("export_rulebook")(self.h, _ptr(ws), _ptr(pairs), _ptr(num), _stream_ptr(stream)))
+        return pairs, num
+
+
+class SubmConv3d(_Conv):
+    kind = "submconv3d"
+
+    def __init__(self, in_channel, out_channel, out_shape_xyz, weights, max_voxels=B.MAX_VOXELS, ksize=3,
+                 stride=1, padding=1, dilation=1):
+        d = D.SubmConv3dDesc()
+        d.in_channel, d.out_channel, d.max_voxels, d.feature_num = in_channel, out_channel, max_voxels, in_channel
+        for a in range(3):
+            d.out_shape[a] = out_shape_xyz[a]
+            d.spatial_shape[a] = out_shape_xyz[a]
+        d.ksize, d.stride, d.padding, d.dilation, d.out_padding = ksize, stride, padding, dilation, 0
+        w = np.ascontiguousarray(weights, np.float32)
+        assert w.shape == (ksize ** 3, in_channel, out_channel)
+        h = C.c_void_p()
+        check(lib().sessd_submconv3d_create(C.byref(d), _np_f32_ptr(w), C.byref(h)))
+        super().__init__(h)
+        self.max_voxels, self.cout, self.kvol = max_voxels, out_channel, ksize ** 3
+
+    def __call__(self, feat, coors, voxel_num, out_dtype=None, stream=None, rulebook_from=None):
+        torch = _torch()
+        out = torch.empty((self.max_voxels, self.cout), dtype=out_dtype or feat.dtype, device=feat.device)
+        ins = [feat, coors, voxel_num]
+        self.configure(ins, [out])
+        if rulebook_from is None:
+            self.enqueue(ins, [out], stream)
+        else:
+            check(lib().sessd_submconv3d_enqueue_shared(self.h, _descs(ins), _descs([out]), _voidpp(ins),
+                                                        _voidpp([out]), _ptr(rulebook_from.ws),
+                                                        _stream_ptr(stream)))
+        return out
+
+
+class SparseConv3d(_Conv):
+    kind = "sparseconv3d"
+
+    def __init__(self, in_channel, out_channel, out_shape_xyz, spatial_shape_xyz, ksize, stride, padding, weights,
+                 max_voxels=B.MAX_VOXELS, dilation=1):
+        d = D.SparseConv3dDesc()
+        d.in_channel, d.out_channel, d.max_voxels, d.feature_num = in_channel, out_channel, max_voxels, in_channel
+        for a in range(3):
+            d.out_shape[a] = out_shape_xyz[a]
+            d.spatial_shape[a] = spatial_shape_xyz[a]
+            d.ksize[a], d.stride[a], d.padding[a] = ksize[a], stride[a], padding[a]
+        d.dilation, d.out_padding = dilation, 0
+        w = np.ascontiguousarray(weights, np.float32)
+        self.kvol = ksize[0] * ksize[1] * ksize[2]
+        assert w.shape == (self.kvol, in_channel, out_channel)
+        h = C.c_void_p()
+        check(lib().sessd_sparseconv3d_create(C.byref(d), _np_f32_ptr(w), C.byref(h)))
+        super().__init__(h)
+        self.max_voxels, self.cout = max_voxels, out_channel
+
+    def __call__(self, feat, coors, voxel_num, out_dtype=None, stream=None):
+        torch = _torch()
+        dev = feat.device
+        out = torch.empty((self.max_voxels, self.cout), dtype=out_dtype or feat.dtype, device=dev)
+        ocoors = torch.empty((self.max_voxels, 4), dtype=torch.int32, device=dev)
+        onum = torch.empty((1,), dtype=torch.int32, device=dev)
+        ins = [feat, coors, voxel_num]
+        self.configure(ins, [out, ocoors, onum])
+        self.enqueue(ins, [out, ocoors, onum], stream)
+        return out, ocoors, onum
+
+
+class Sparse2Dense(_Plugin):
+    kind = "sparse2dense"
+
+    def __init__(self, feature_map_size_xyz=B.DENSE_SIZE_XYZ, feature_map_channel=B.DENSE_CHANNEL):
+        d = B.dense_desc(feature_map_size_xyz, feature_map_channel)
+        h = C.c_void_p()
+        check(lib().sessd_sparse2dense_create(C.byref(d), C.byref(h)))
+        super().__init__(h)
+        self.size, self.channel = tuple(feature_map_size_xyz), feature_map_channel
+
+    def __call__(self, feat, coors, voxel_num, out_dtype=None, stream=None):
+        torch = _torch()
+        W, H, Dz = self.size
+        dense = torch.empty((self.channel * Dz, H, W), dtype=out_dtype or feat.dtype, device=feat.device)
+        ins = [feat, coors, voxel_num]
+        self.configure(ins, [dense])
+        self.enqueue(ins, [dense], stream)
+        return dense
+
+    def status(self, stream=None):
+        torch = _torch()
+        torch.cuda.synchronize()
+        return int(self.ws[:4].view(torch.int32)[0].item())
+
+
+def make_conv(layer: B.Layer, weights, prev_grid_xyz, max_voxels, scale=None, shift=None, relu=True):
+    """Plugin for one entry of the backbone table, with its folded BatchNorm + ReLU epilogue."""
+    if layer.type == D.SESSD_LAYER_SUBM:
+        p = SubmConv3d(layer.cin, layer.cout, layer.out_shape, weights, max_voxels, layer.ksize[0],
+                       layer.stride[0], layer.padding[0])
+    else:
+        p = SparseConv3d(layer.cin, layer.cout, layer.out_shape, prev_grid_xyz, layer.ksize, layer.stride,
+                         layer.padding, weights, max_voxels)
+    if scale is not None or shift is not None or relu:
+        p.set_epilogue(scale, shift, relu)
+    return p
+
+
+class Pipeline:
+    """voxelGenerator -> conv stack -> sparse2Dense, owned and run by the library (C++)."""
+
+    def __init__(self, layers, weights: B.Weights, max_points, max_voxels=B.MAX_VOXELS, point_features=4,
+                 feature_dtype="fp32", relu=True, share_rulebooks=True, skip_pad_rows=False, use_graph=False,
+                 dense_size_xyz=B.DENSE_SIZE_XYZ, max_pts_per_voxel=B.MAX_NUM_POINTS_PER_VOXEL,
+                 use_epilogue=True):
+        torch = _torch()
+        self.layers = list(layers)
+        self.max_points, self.max_voxels = max_points, max_voxels
+        self.dtype = torch.float16 if feature_dtype in ("fp16", "half", torch.float16) else torch.float32
+        n = len(self.layers)
+        self._specs = B.layer_specs(self.layers)
+        self._w = [np.ascontiguousarray(w, np.float32) for w in weights.w]
+        self._s = [np.ascontiguousarray(s, np.float32) for s in weights.scale]
+        self._b = [np.ascontiguousarray(s, np.float32) for s in weights.shift]
+        FP = C.POINTER(C.c_float)
+        arr = lambda xs: (FP * max(n, 1))(*[x.ctypes.data_as(FP) for x in xs])  # noqa: E731
+        d = D.PipelineDesc()
+        d.voxelgen = B.voxelgen_desc(max_voxels, max_pts_per_voxel)
+        d.max_points, d.point_features, d.n_layers = max_points, point_features, n
+        d.layers = self._specs
+        d.weights = arr(self._w)
+        if use_epilogue:
+            d.scale = arr(self._s)
+            d.shift = arr(self._b)
+        d.relu = int(relu)
+        d.feature_dtype = D.SESSD_HALF if self.dtype == torch.float16 else D.SESSD_FLOAT
+        c_last = self.layers[-1].cout if n else 4
+        d.dense = B.dense_desc(dense_size_xyz, c_last)
+        d.share_rulebooks = int(share_rulebooks)
+        d.flags = D.SESSD_FLAG_SKIP_PAD_ROWS if skip_pad_rows else 0
+        d.use_graph = int(use_graph)
+        self.dense_shape = (c_last * dense_size_xyz[2], dense_size_xyz[1], dense_size_xyz[0])
+        self.h = C.c_void_p()
+        check(lib().sessd_pipeline_create(C.byref(d), C.byref(self.h)))
+
+    def new_dense(self, device="cuda"):
+        torch = _torch()
+        return torch.empty(self.dense_shape, dtype=self.dtype, device=device)
+
+    def enqueue(self, points, points_size, dense, stream=None):
+        check(lib().sessd_pipeline_enqueue(self.h, _ptr(points), _ptr(points_size), _ptr(dense), _stream_ptr(stream)))
+
+    def layer_io(self, layer):
+        """-> (feat ptr, coors ptr, voxel_num ptr, workspace ptr, channels) of layer (or -1 = voxelizer)"""
+        f, c, n, w = C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_void_p()
+        ch = C.c_int32()
+        check(lib().sessd_pipeline_layer_io(self.h, layer, C.byref(f), C.byref(c), C.byref(n), C.byref(w), C.byref(ch)))
+        return f.value, c.value, n.value, w.value, ch.value
+
+    def read_layer(self, layer):
+        """Copy a layer's output of the last enqueue to the host: feat[n,C] float32, coors[n,4], n."""
+        torch = _torch()
+        torch.cuda.synchronize()
+        f, c, n, _, ch = self.layer_io(layer)
+        num = np.zeros(1, np.int32)
+        _hip_d2h(num, n)
+        cnt = int(num[0])
+        es = 4 if (layer < 0 or self.dtype == torch.float32) else 2
+        feat = np.zeros((self.max_voxels, ch), np.float32 if es == 4 else np.float16)
+        coors = np.zeros((self.max_voxels, 4), np.int32)
+        _hip_d2h(feat, f)
+        _hip_d2h(coors, c)
+        return feat[:cnt].astype(np.float32), coors[:cnt], cnt
+
+    def status(self, stream=None):
+        s = C.c_int32(0)
+        check(lib().sessd_pipeline_status(self.h, _stream_ptr(stream), C.byref(s)))
+        return s.value
+
+    def device_bytes(self):
+        return lib().sessd_pipeline_device_bytes(self.h)
+
+    def num_launches(self):
+        return lib().sessd_pipeline_num_launches(self.h)
+
+    def close(self):
+        if self.h:
+            lib().sessd_pipeline_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+_hip = None
+
+
+def _hip_d2h(dst_np, src_ptr):
+    """hipMemcpy device->host into a numpy array (for pointers owned by the library)."""
+    global _hip
+    if _hip is None:
+        _hip = C.CDLL("libamdhip64.so")
+        _hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+    rc = _hip.hipMemcpy(dst_np.ctypes.data_as(C.c_void_p), C.c_void_p(src_ptr), dst_np.nbytes, 2)
+    if rc != 0:
+        raise SessdError("hipMemcpy D2H failed: %d" % rc)

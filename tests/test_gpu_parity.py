@@ -1,0 +1,329 @@
+"""GPU parity: every plugin of libsessd3d, called through the C-ABI, against the CPU oracle on the same
+seeded inputs.  Integer results (voxel coordinates, active sites, rulebooks, counts) must be
+bit-exact, after canonical sort where the numbering is free; FP32 features within 1e-4 relative."""
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as O
+from gpu_util import (DEV, RTOL_FP32, assert_features_close, canonical, dev, points_input, to_np)
+from sessd3d import api, backbone as B, ctypes_defs as D, frames as F
+
+pytestmark = pytest.mark.gpu
+
+RANGE, VSIZE = B.POINT_CLOUD_RANGE, B.VOXEL_SIZE
+
+
+def run_voxelgen(pts, max_points, max_voxels, max_pts=5):
+    vg = api.VoxelGenerator(max_voxels=max_voxels, max_num_points_per_voxel=max_pts)
+    p, n = points_input(pts, max_points)
+    vox, coors, num = vg(p, n)
+    torch.cuda.synchronize()
+    return to_np(vox), to_np(coors), int(to_np(num)[0]), vg.status()
+
+
+def check_voxelgen(pts, max_points, max_voxels, max_pts=5):
+    vox, coors, n, st = run_voxelgen(pts, max_points, max_voxels, max_pts)
+    o_vox, o_coors, o_n, _, o_st = O.voxelize(pts[:max_points], RANGE, VSIZE, max_pts, max_voxels)
+    assert n == o_n
+    assert st == o_st
+    # same numbering (first appearance) -> comparable row by row, and again after canonical sort
+    assert np.array_equal(coors, o_coors)
+    assert np.array_equal(vox.view(np.uint32), o_vox.view(np.uint32))      # bit-exact means
+    a = canonical(coors, n, vox)
+    b = canonical(o_coors, o_n, o_vox)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    return n
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_voxelgen_config2(seed):
+    """BASELINE config 2: 20 000 points, voxel 0.05x0.05x0.1, <= 5 points/voxel, cap 20 000."""
+    pts = F.lidar_frame(20000, seed)
+    n = check_voxelgen(pts, 20000, 20000)
+    assert 14000 < n <= 20000
+
+
+def test_voxelgen_reference_shapes_and_padding():
+    """MAX_POINTS 80000 / MAX_VOXELS 60000 as in params.h; rows past points_size are ignored even if
+    they hold in-range garbage."""
+    pts = F.lidar_frame(20000, 2)
+    vg = api.VoxelGenerator(max_voxels=60000)
+    buf = np.tile(pts[:100], (800, 1)).astype(np.float32)      # 80000 rows of valid-looking points
+    buf[:20000] = pts
+    vox, coors, num = vg(dev(buf), dev(np.array([20000], np.int32)))
+    torch.cuda.synchronize()
+    o = O.voxelize(pts, RANGE, VSIZE, 5, 60000)
+    assert int(to_np(num)[0]) == o[2]
+    assert np.array_equal(to_np(coors), o[1]) and np.array_equal(to_np(vox).view(np.uint32), o[0].view(np.uint32))
+    assert vg.status() == 0
+
+
+def test_voxelgen_crowded_voxels_and_shuffled_order():
+    rng = np.random.default_rng(3)
+    pts = F.lidar_frame(12000, 3)
+    extra = pts[rng.integers(0, len(pts), 6000)] + rng.normal(0, 0.004, (6000, 4)).astype(np.float32)
+    pts = np.concatenate([pts, extra.astype(np.float32)])[rng.permutation(18000)]
+    check_voxelgen(pts, 18000, 20000)
+    check_voxelgen(pts, 18000, 20000, max_pts=3)
+    check_voxelgen(pts, 18000, 20000, max_pts=8)
+
+
+def test_voxelgen_cap_overflow_and_edges():
+    pts = F.lidar_frame(20000, 4)
+    check_voxelgen(pts, 20000, 5000)                 # cap binds: first 5000 cells kept, flag raised
+    vox, coors, n, st = run_voxelgen(pts, 20000, 5000)
+    assert n == 5000 and st & D.SESSD_STATUS_VOXEL_OVERFLOW
+    check_voxelgen(pts[:0], 1024, 1000)              # empty cloud
+    check_voxelgen(pts[:1], 1024, 1000)
+    # points_size larger than the tensor: clamped to max_points
+    vox, coors, n, st = run_voxelgen(pts, 4096, 20000)
+    assert n == O.voxelize(pts[:4096], RANGE, VSIZE, 5, 20000)[2]
+    f = np.float32
+    below = lambda v: np.nextafter(f(v), f(-np.inf))   # noqa: E731
+    edge = np.array([[0.0, -40.0, -3.0, 0.1], [70.4, 0.0, 0.0, 0.2], [10.0, 40.0, 0.0, 0.3], [10.0, 0.0, 1.0, 0.4],
+                     [10.0, 0.0, below(1.0), 0.5], [10.0, below(40.0), 0.0, 0.6], [below(70.4), 0.0, 0.0, 0.7],
+                     [-0.0, 0.0, 0.0, 0.8], [np.nan, 0.0, 0.0, 0.9], [np.inf, 0.0, 0.0, 1.0]], np.float32)
+    assert check_voxelgen(edge, 64, 100) == 3
+
+
+def test_voxelgen_five_point_features():
+    pts = F.lidar_frame(8000, 5)
+    pts5 = np.concatenate([pts, np.full((8000, 1), 7.0, np.float32)], axis=1)
+    check_voxelgen(pts5, 8192, 20000)
+
+
+def run_subm(coors_np, n, feat_np, w, grid_zyx, max_voxels, scale=None, shift=None, relu=False):
+    conv = api.SubmConv3d(w.shape[1], w.shape[2], grid_zyx[::-1], w, max_voxels)
+    if scale is not None or relu:
+        conv.set_epilogue(scale, shift, relu)
+    cbuf = np.zeros((max_voxels, 4), np.int32)
+    cbuf[:n] = coors_np[:n]
+    fbuf = np.zeros((max_voxels, w.shape[1]), np.float32)
+    fbuf[:n] = feat_np[:n]
+    out = conv(dev(fbuf), dev(cbuf), dev(np.array([n], np.int32)))
+    pairs, num = conv.export_rulebook()
+    torch.cuda.synchronize()
+    return conv, to_np(out), to_np(pairs), to_np(num).astype(np.uint32), cbuf
+
+
+def test_subm_config1_rulebook_and_features():
+    """BASELINE config 1: one SubMConv3d 4->16 on 2000 uniform voxels in 41x160x140."""
+    grid = (41, 160, 140)
+    n, mv = 2000, 2000
+    rng = np.random.default_rng(0)
+    coors = F.random_active_voxels(n, grid, 0)
+    feat = rng.uniform(0, 1, (n, 4)).astype(np.float32)
+    w = rng.normal(0, 0.1, (27, 4, 16)).astype(np.float32)
+    conv, out, pairs, num, cbuf = run_subm(coors, n, feat, w, grid, mv)
+    o_pairs, o_num, _ = O.subm_rulebook(coors, n, grid[::-1], mv)
+    assert np.array_equal(num, o_num)
+    assert np.array_equal(O.canonical_rulebook(pairs, num, cbuf, cbuf), O.canonical_rulebook(o_pairs, o_num, coors, coors))
+    o_out = O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv)
+    assert_features_close(out, o_out, RTOL_FP32, "subm config 1")
+    assert conv.status() == 0
+
+
+@pytest.mark.parametrize("cin,cout", [(4, 16), (16, 16), (32, 32), (64, 64), (5, 7)])
+def test_subm_clustered_with_epilogue_and_pad_rows(cin, cout):
+    grid = (21, 200, 176)
+    n, mv = 6000, 8192
+    rng = np.random.default_rng(cin)
+    coors = F.clustered_active_voxels(n, grid, 1, n_blobs=60)
+    feat = rng.uniform(-1, 1, (n, cin)).astype(np.float32)
+    w = rng.normal(0, 0.1, (27, cin, cout)).astype(np.float32)
+    sc = rng.uniform(0.5, 1.5, cout).astype(np.float32)
+    sh = rng.uniform(-0.2, 0.2, cout).astype(np.float32)
+    conv, out, pairs, num, cbuf = run_subm(coors, n, feat, w, grid, mv, sc, sh, True)
+    o_pairs, o_num, _ = O.subm_rulebook(coors, n, grid[::-1], mv)
+    assert int(o_num.sum()) > 4 * n
+    assert np.array_equal(num, o_num)
+    assert np.array_equal(O.canonical_rulebook(pairs, num, cbuf, cbuf), O.canonical_rulebook(o_pairs, o_num, coors, coors))
+    # within an offset the exported pairs are in ascending output-row order, unused entries are -1
+    for k in (0, 13, 26):
+        assert np.all(np.diff(pairs[k, 1, :num[k]]) > 0) and np.all(pairs[k, :, num[k]:] == -1)
+    o_out = O.scale_shift_relu(O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), mv, sc, sh, True)
+    assert_features_close(out, o_out, RTOL_FP32, "subm %d->%d" % (cin, cout))   # incl. pad rows = relu(shift)
+
+
+def test_subm_shared_rulebook_skip_pad_and_empty():
+    grid = (11, 100, 88)
+    n, mv = 3000, 4096
+    rng = np.random.default_rng(5)
+    coors = F.clustered_active_voxels(n, grid, 2)
+    feat = rng.uniform(-1, 1, (n, 16)).astype(np.float32)
+    w1 = rng.normal(0, 0.1, (27, 16, 16)).astype(np.float32)
+    w2 = rng.normal(0, 0.1, (27, 16, 32)).astype(np.float32)
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = np.zeros((mv, 16), np.float32)
+    fbuf[:n] = feat
+    a = api.SubmConv3d(16, 16, grid[::-1], w1, mv)
+    b = api.SubmConv3d(16, 32, grid[::-1], w2, mv)
+    b.set_flags(D.SESSD_FLAG_SKIP_PAD_ROWS)
+    d_coors, d_num = dev(cbuf), dev(np.array([n], np.int32))
+    y1 = a(dev(fbuf), d_coors, d_num)
+    y2 = b(y1, d_coors, d_num, rulebook_from=a)           # GEMM only, on a's rulebook
+    torch.cuda.synchronize()
+    o_pairs, o_num, _ = O.subm_rulebook(coors, n, grid[::-1], mv)
+    o1 = O.gather_gemm_scatter(feat, w1, o_pairs, o_num, mv)
+    o2 = O.gather_gemm_scatter(o1, w2, o_pairs, o_num, mv)
+    assert_features_close(to_np(y1), o1, RTOL_FP32, "shared: layer 1")
+    assert_features_close(to_np(y2)[:n], o2[:n], RTOL_FP32, "shared: layer 2")
+    # empty input: nothing active, all rows are pad rows
+    y0 = a(dev(fbuf), d_coors, dev(np.array([0], np.int32)))
+    pairs, num = a.export_rulebook()
+    torch.cuda.synchronize()
+    assert np.all(to_np(y0) == 0) and np.all(to_np(num) == 0) and np.all(to_np(pairs) == -1)
+
+
+def test_subm_bad_coordinate_is_flagged_not_written():
+    grid = (5, 20, 20)
+    coors = np.array([[0, 1, 1, 1], [0, 1, 1, 2], [0, 7, 1, 1], [0, 1, 25, 1]], np.int32)   # rows 2,3 outside
+    feat = np.ones((4, 4), np.float32)
+    w = np.ones((27, 4, 4), np.float32)
+    conv, out, pairs, num, _ = run_subm(coors, 4, feat, w, grid, 64)
+    assert conv.status() & D.SESSD_STATUS_BAD_COORD
+    o_pairs, o_num, o_st = O.subm_rulebook(coors, 4, grid[::-1], 64)
+    assert o_st & D.SESSD_STATUS_BAD_COORD and np.array_equal(num, o_num)
+    assert np.array_equal(out, O.gather_gemm_scatter(feat, w, o_pairs, o_num, 64))
+
+
+SPARSE_LAYERS = [l for l in B.reference_layers() if l.type == D.SESSD_LAYER_SPARSE]
+
+
+def sparse_input_grid(layer):
+    """Input grid (z,y,x) of a reference sparse layer = out grid of the stage before it."""
+    prev = {"sparse6": (41, 1600, 1408), "sparse15": (21, 800, 704), "sparse27": (11, 400, 352), "sparse39": (5, 200, 176)}
+    return prev[layer.name]
+
+
+def run_sparse(layer, coors, n, feat, w, mv, in_grid_zyx, **kw):
+    conv = api.SparseConv3d(layer.cin, layer.cout, layer.out_shape, in_grid_zyx[::-1], layer.ksize, layer.stride,
+                            layer.padding, w, mv)
+    if kw.get("epilogue"):
+        conv.set_epilogue(*kw["epilogue"])
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors[:n]
+    fbuf = np.zeros((mv, layer.cin), np.float32)
+    fbuf[:n] = feat[:n]
+    out, oc, on = conv(dev(fbuf), dev(cbuf), dev(np.array([n], np.int32)))
+    pairs, num = conv.export_rulebook()
+    torch.cuda.synchronize()
+    return conv, to_np(out), to_np(oc), int(to_np(on)[0]), to_np(pairs), to_np(num).astype(np.uint32)
+
+
+@pytest.mark.parametrize("layer", SPARSE_LAYERS, ids=[l.name for l in SPARSE_LAYERS])
+def test_sparse_layers_of_the_backbone(layer):
+    """Each strided layer shape of params.h on a neighbour-rich active set in its own input grid."""
+    ig = sparse_input_grid(layer)
+    n, mv = 5000, 30000
+    rng = np.random.default_rng(len(layer.name))
+    sub = (ig[0], min(ig[1], 300), min(ig[2], 300))
+    coors = F.clustered_active_voxels(n, sub, 3, n_blobs=50)
+    feat = rng.uniform(-1, 1, (n, layer.cin)).astype(np.float32)
+    w = rng.normal(0, 0.1, (layer.kvol, layer.cin, layer.cout)).astype(np.float32)
+    conv, out, oc, on, pairs, num = run_sparse(layer, coors, n, feat, w, mv, ig)
+    o_pairs, o_num, o_oc, o_on, o_st = O.sparse_rulebook(coors, n, layer.out_shape, layer.ksize, layer.stride,
+                                                         layer.padding, mv)
+    assert on == o_on and conv.status() == o_st == 0
+    assert np.array_equal(oc, o_oc)                       # first-seen numbering reproduced row by row
+    assert np.array_equal(canonical(oc, on)[0], canonical(o_oc, o_on)[0])
+    assert np.array_equal(num, o_num)
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    assert np.array_equal(O.canonical_rulebook(pairs, num, cbuf, oc), O.canonical_rulebook(o_pairs, o_num, coors, o_oc))
+    o_out = O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv)
+    assert_features_close(out, o_out, RTOL_FP32, layer.name)
+    a = canonical(oc, on, out)
+    b = canonical(o_oc, o_on, o_out)
+    assert_features_close(a[1], b[1], RTOL_FP32, layer.name + " (canonical order)")
+
+
+def test_sparse_cap_overflow_and_empty():
+    layer = SPARSE_LAYERS[0]
+    ig = sparse_input_grid(layer)
+    n = 4000
+    rng = np.random.default_rng(9)
+    coors = F.random_active_voxels(n, (ig[0], 200, 200), 4)    # uncorrelated sites: the set grows ~8x
+    feat = rng.uniform(-1, 1, (n, layer.cin)).astype(np.float32)
+    w = rng.normal(0, 0.1, (layer.kvol, layer.cin, layer.cout)).astype(np.float32)
+    mv = 8192
+    conv, out, oc, on, pairs, num = run_sparse(layer, coors, n, feat, w, mv, ig)
+    o_pairs, o_num, o_oc, o_on, o_st = O.sparse_rulebook(coors, n, layer.out_shape, layer.ksize, layer.stride,
+                                                         layer.padding, mv)
+    assert o_st & D.SESSD_STATUS_VOXEL_OVERFLOW and conv.status() & D.SESSD_STATUS_VOXEL_OVERFLOW
+    assert on == o_on == mv and np.array_equal(oc, o_oc) and np.array_equal(num, o_num)
+    assert_features_close(out, O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), RTOL_FP32, "capped sparse layer")
+    conv, out, oc, on, pairs, num = run_sparse(layer, coors, 0, feat, w, mv, ig)
+    assert on == 0 and np.all(out == 0) and np.all(oc == 0) and np.all(num == 0)
+
+
+def test_sparse_generic_stride1_and_corner_truncation():
+    """stride 1 (27 candidates per input) and cells at coordinate 0 with padding 0 (C division
+    truncates toward zero in getValidOutPos)."""
+    cases = [((3, 3, 3), (1, 1, 1), (1, 1, 1), (6, 9, 8)), ((3, 3, 3), (2, 2, 2), (0, 0, 0), (9, 9, 9)),
+             ((2, 2, 2), (2, 2, 2), (0, 0, 0), (8, 8, 8)), ((1, 3, 3), (1, 2, 2), (0, 1, 1), (4, 9, 9))]
+    rng = np.random.default_rng(1)
+    for k, s, p, ig in cases:
+        og = tuple(B.conv_out_size(ig[a], k[a], s[a], p[a]) for a in range(3))
+        layer = B.Layer("t", D.SESSD_LAYER_SPARSE, 8, 16, og[::-1], k, s, p)
+        n = ig[0] * ig[1] * ig[2] // 2
+        coors = F.random_active_voxels(n, ig, 6)
+        feat = rng.uniform(-1, 1, (n, 8)).astype(np.float32)
+        w = rng.normal(0, 0.1, (layer.kvol, 8, 16)).astype(np.float32)
+        mv = 1024
+        conv, out, oc, on, pairs, num = run_sparse(layer, coors, n, feat, w, mv, ig)
+        o_pairs, o_num, o_oc, o_on, _ = O.sparse_rulebook(coors, n, og[::-1], k, s, p, mv)
+        assert on == o_on and np.array_equal(oc, o_oc) and np.array_equal(num, o_num), (k, s, p)
+        assert_features_close(out, O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), RTOL_FP32, str((k, s, p)))
+
+
+def test_sparse2dense():
+    rng = np.random.default_rng(2)
+    n, mv, c = 2739, 60000, 64
+    coors = F.random_active_voxels(n, (2, 200, 176), 8)
+    feat = rng.uniform(0.1, 1, (n, c)).astype(np.float32)
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = rng.uniform(5, 6, (mv, c)).astype(np.float32)      # rows >= n hold garbage that must not leak
+    fbuf[:n] = feat
+    s2d = api.Sparse2Dense()
+    dense = s2d(dev(fbuf), dev(cbuf), dev(np.array([n], np.int32)))
+    torch.cuda.synchronize()
+    want = O.sparse2dense(feat, coors, n, B.DENSE_SIZE_XYZ)
+    assert dense.shape == (128, 200, 176)
+    assert np.array_equal(to_np(dense), want)
+    assert s2d.status() == 0
+    # idempotent on a dirty output buffer, empty input gives all zeros
+    dense.fill_(3.0)
+    s2d.enqueue([dev(fbuf), dev(cbuf), dev(np.array([0], np.int32))], [dense])
+    torch.cuda.synchronize()
+    assert float(dense.abs().max()) == 0.0
+    cbuf[5] = (0, 2, 0, 0)                                        # z outside D=2
+    s2d(dev(fbuf), dev(cbuf), dev(np.array([n], np.int32)))
+    assert s2d.status() & D.SESSD_STATUS_BAD_COORD
+
+
+def test_conv_serialization_round_trip():
+    rng = np.random.default_rng(4)
+    w = rng.normal(0, 0.1, (27, 4, 16)).astype(np.float32)
+    a = api.SubmConv3d(4, 16, (140, 160, 41), w, 2000)
+    blob = a.serialize()
+    assert len(blob) == 16 * 4 + w.size * 4                     # submConv3dlayer.cu:684-687
+    head = np.frombuffer(blob[:64], np.int32)
+    assert head.tolist() == [4, 16, 2000, 4, 140, 160, 41, 140, 160, 41, 3, 1, 1, 1, 0, w.size]
+    assert np.array_equal(np.frombuffer(blob[64:], np.float32), w.ravel())
+    a.set_epilogue(np.ones(16), np.zeros(16), True)
+    blob2 = a.serialize()
+    assert blob2[:len(blob)] == blob and len(blob2) > len(blob)
+    b = api.SubmConv3d.deserialize(blob2)
+    assert b.serialize() == blob2
+    layer = SPARSE_LAYERS[2]
+    ws = rng.normal(0, 0.1, (27, 64, 64)).astype(np.float32)
+    s = api.SparseConv3d(64, 64, layer.out_shape, (352, 400, 11), layer.ksize, layer.stride, layer.padding, ws, 60000)
+    sb = s.serialize()
+    assert len(sb) == 22 * 4 + ws.size * 4                      # sparseConv3dlayer.cu:863-866
+    assert np.frombuffer(sb[:88], np.int32).tolist() == [64, 64, 60000, 64, 176, 200, 5, 352, 400, 11, 3, 3, 3,
+                                                          2, 2, 2, 0, 1, 1, 1, 0, ws.size]
+    assert api.SparseConv3d.deserialize(sb).serialize() == sb

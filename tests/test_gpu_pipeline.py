@@ -1,0 +1,104 @@
+"""GPU parity of the whole frame pipeline (voxelGenerator -> 14 conv layers with folded BN + ReLU ->
+sparse2Dense) against oracle_frame, plus size-independent properties at the full benchmark size."""
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as O
+from gpu_util import RTOL_FP32, assert_features_close, canonical, points_input, to_np
+from sessd3d import api, backbone as B, ctypes_defs as D, frames as F
+
+pytestmark = pytest.mark.gpu
+
+
+def run_pipeline(pts, layers, W, max_points, max_voxels, **kw):
+    pipe = api.Pipeline(layers, W, max_points, max_voxels, **kw)
+    p, n = points_input(pts, max_points)
+    dense = pipe.new_dense()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        pipe.enqueue(p, n, dense, stream)
+    stream.synchronize()
+    return pipe, dense, (p, n, stream)
+
+
+def compare_with_oracle(pipe, dense, pts, layers, W, max_voxels, rtol):
+    ref = O.frame(pts, B.voxelgen_desc(max_voxels=max_voxels), layers, W, B.dense_desc())
+    counts = [pipe.read_layer(l)[2] for l in range(-1, len(layers))]
+    assert counts == ref["counts"].tolist()
+    feat, coors, n = pipe.read_layer(len(layers) - 1)
+    assert np.array_equal(coors, ref["coors"])                       # same numbering, row by row
+    a, b = canonical(coors, n, feat), canonical(ref["coors"], n, ref["feat"])
+    assert np.array_equal(a[0], b[0])
+    assert_features_close(a[1], b[1], rtol, "last layer features")
+    assert_features_close(to_np(dense).astype(np.float32), ref["dense"], rtol, "dense BEV tensor")
+    assert pipe.status() == ref["status"]
+    return ref
+
+
+@pytest.mark.parametrize("share,skip_pad", [(True, True), (False, False)])
+def test_full_backbone_small_frame(share, skip_pad):
+    pts = F.lidar_frame(5000, 11)
+    layers = B.reference_layers()
+    W = B.random_weights(layers, seed=5, w_std=0.05)
+    pipe, dense, _ = run_pipeline(pts, layers, W, 8192, 16384, share_rulebooks=share, skip_pad_rows=skip_pad)
+    compare_with_oracle(pipe, dense, pts, layers, W, 16384, RTOL_FP32)
+
+
+def test_full_backbone_config3_frame_and_graph_replay():
+    """BASELINE config 3: the 20 000-point frame (~17 k voxels) through the reference's 14 conv layers.
+    The eager enqueue and repeated replays of the captured graph must give identical bits."""
+    pts = F.lidar_frame(20000, 0)
+    layers = B.reference_layers()
+    W = B.random_weights(layers, seed=1, w_std=0.05)
+    pipe, dense, _ = run_pipeline(pts, layers, W, 20000, 60000, share_rulebooks=True, skip_pad_rows=True)
+    ref = compare_with_oracle(pipe, dense, pts, layers, W, 60000, RTOL_FP32)
+    assert 15000 < ref["counts"][0] < 19000
+    eager = to_np(dense).copy()
+
+    gpipe = api.Pipeline(layers, W, 20000, 60000, share_rulebooks=True, skip_pad_rows=True, use_graph=True)
+    p, n = points_input(pts, 20000)
+    gd = gpipe.new_dense()
+    stream = torch.cuda.Stream()
+    for rep in range(3):
+        gd.fill_(float(rep + 1))                        # eager work between replays
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            gpipe.enqueue(p, n, gd, stream)
+        stream.synchronize()
+        assert np.array_equal(to_np(gd), eager), "graph replay %d differs from the eager result" % rep
+    assert gpipe.num_launches() > 0
+    # a different frame in the same buffers: the replayed graph reads the new data
+    pts2 = F.lidar_frame(18000, 1)
+    p2, n2 = points_input(pts2, 20000)
+    p.copy_(p2)
+    n.copy_(n2)
+    with torch.cuda.stream(stream):
+        gpipe.enqueue(p, n, gd, stream)
+    stream.synchronize()
+    ref2 = O.frame(pts2, B.voxelgen_desc(max_voxels=60000), layers, W, B.dense_desc())
+    assert_features_close(to_np(gd), ref2["dense"], RTOL_FP32, "graph replay on a new frame")
+
+
+def test_properties_at_full_size():
+    """Size-independent checks on a frame too large to push through the CPU oracle quickly:
+    determinism, active-site bookkeeping and dense/sparse consistency."""
+    pts = F.lidar_frame(60000, 7)
+    layers = B.reference_layers()
+    W = B.random_weights(layers, seed=2, w_std=0.05)
+    pipe, dense, (p, n, stream) = run_pipeline(pts, layers, W, 60000, 60000, skip_pad_rows=True)
+    first = to_np(dense).copy()
+    with torch.cuda.stream(stream):
+        pipe.enqueue(p, n, dense, stream)
+    stream.synchronize()
+    assert np.array_equal(to_np(dense), first)                     # run-to-run bit identical
+    feat, coors, cnt = pipe.read_layer(len(layers) - 1)
+    assert len(np.unique(coors[:, 1:] @ np.array([200 * 176, 176, 1]))) == cnt     # unique sites
+    assert coors[:, 1].max() < 2 and coors[:, 2].max() < 200 and coors[:, 3].max() < 176 and coors.min() >= 0
+    back = first.reshape(64, 2, 200, 176)[:, coors[:, 1], coors[:, 2], coors[:, 3]].T
+    assert np.array_equal(back, feat)                               # dense holds exactly the sparse rows
+    assert np.count_nonzero(first) == np.count_nonzero(feat)
+    # voxelizer output is independent of everything downstream: compare with the oracle's voxelizer
+    vfeat, vcoors, vn = pipe.read_layer(-1)
+    o = O.voxelize(pts, B.POINT_CLOUD_RANGE, B.VOXEL_SIZE, 5, 60000)
+    assert vn == o[2] and np.array_equal(vcoors, o[1][:vn]) and np.array_equal(vfeat.view(np.uint32), o[0][:vn].view(np.uint32))

@@ -1,0 +1,118 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every declared symbol, and the host logic
+that needs no GPU (descriptors, serialisation, grid derivation, argument checking) behaves like the
+reference plugins.  No kernel is launched here."""
+import ctypes as C
+import struct
+
+import numpy as np
+import pytest
+
+from sessd3d import api, backbone as B, ctypes_defs as D
+
+
+def test_library_exports_every_declared_symbol():
+    L = api.lib()
+    names = api.declared_symbols()
+    assert len(names) >= 50
+    missing = [n for n in names if not hasattr(L, n)]
+    assert not missing, missing
+    assert b"gfx950" in L.sessd_version()
+
+
+def test_struct_layouts_match_header_sizes():
+    assert C.sizeof(D.TensorDesc) == 4 + 32 + 4 + 4 + 4
+    assert C.sizeof(D.VoxelGenDesc) == 4 + 4 + 24 + 4 + 12
+    assert C.sizeof(D.SubmConv3dDesc) == 4 * 4 + 12 + 12 + 5 * 4
+    assert C.sizeof(D.SparseConv3dDesc) == 4 * 4 + 12 * 5 + 2 * 4
+    assert C.sizeof(D.Sparse2DenseDesc) == 16
+    assert C.sizeof(D.LayerSpec) == 12 + 12 * 4
+
+
+def test_reference_backbone_table_matches_python_table():
+    L = api.lib()
+    specs = (D.LayerSpec * 14)()
+    vg, dd = D.VoxelGenDesc(), D.Sparse2DenseDesc()
+    assert L.sessd_reference_backbone(specs, 14, C.byref(vg), C.byref(dd)) == 14
+    for s, l in zip(specs, B.reference_layers()):
+        assert (s.type, s.in_channel, s.out_channel) == (l.type, l.cin, l.cout)
+        assert tuple(s.ksize) == l.ksize and tuple(s.stride) == l.stride and tuple(s.padding) == l.padding
+        assert tuple(s.out_shape) == l.out_shape
+    assert vg.max_voxels == 60000 and vg.max_num_points_per_voxel == 5
+    assert np.allclose(list(vg.point_cloud_range), B.POINT_CLOUD_RANGE) and np.allclose(list(vg.voxel_size), B.VOXEL_SIZE)
+    assert tuple(dd.feature_map_size) == (176, 200, 2) and dd.feature_map_channel == 64
+    # each sparse layer's out grid follows from the previous grid (spconv formula)
+    g = (1408, 1600, 41)
+    for l in B.reference_layers():
+        if l.type == D.SESSD_LAYER_SPARSE:
+            g = tuple(B.conv_out_size(g[a], l.ksize[2 - a], l.stride[2 - a], l.padding[2 - a]) for a in range(3))
+        assert l.out_shape == g
+
+
+def test_voxelgen_host_side():
+    vg = api.VoxelGenerator(max_voxels=20000)
+    blob = vg.serialize()
+    # voxelGenerator.cu:584-599: 3 ints, 9 floats, 4 ints
+    assert len(blob) == 7 * 4 + 9 * 4
+    f = struct.unpack("<3i9f4i", blob)
+    assert f[:3] == (20000, 5, 4)
+    assert np.allclose(f[3:12], [0.0, 70.4, -40.0, 40.0, -3.0, 1.0, 0.05, 0.05, 0.1])
+    assert f[13:] == (1408, 1600, 40)          # grid derived at create, as configurePlugin would
+    assert vg.grid_size() == (1408, 1600, 40)
+    vg2 = api.VoxelGenerator.deserialize(blob)
+    assert vg2.serialize() == blob
+    ind = (D.TensorDesc * 2)(D.TensorDesc.make([1, 80000, 4], D.SESSD_FLOAT), D.TensorDesc.make([1], D.SESSD_INT32))
+    outd = (D.TensorDesc * 3)(D.TensorDesc.make([1, 20000, 4], D.SESSD_FLOAT),
+                              D.TensorDesc.make([1, 20000, 4], D.SESSD_INT32), D.TensorDesc.make([1], D.SESSD_INT32))
+    L = api.lib()
+    assert L.sessd_voxelgen_configure(vg.h, ind, 2, outd, 3) == 0
+    ws = L.sessd_voxelgen_workspace_size(vg.h, ind, 2, outd, 3)
+    # hash table instead of the reference's 721 MB dense slot table
+    assert 0 < ws < 16 * 2 ** 20
+    # enqueue argument checking happens before any launch
+    assert L.sessd_voxelgen_enqueue(vg.h, ind, outd, None, None, None, None) == D.SESSD_E_INVALID
+    assert b"null" in L.sessd_last_error()
+
+
+def test_voxelgen_create_rejects_bad_fields():
+    L = api.lib()
+    d = B.voxelgen_desc()
+    d.voxel_size[1] = 0.0
+    h = C.c_void_p()
+    assert L.sessd_voxelgen_create(C.byref(d), C.byref(h)) == D.SESSD_E_INVALID
+    d = B.voxelgen_desc()
+    d.voxel_feature_num = 5
+    assert L.sessd_voxelgen_create(C.byref(d), C.byref(h)) == D.SESSD_E_UNSUPPORTED
+    assert L.sessd_voxelgen_deserialize(b"\0" * 10, 10, C.byref(h)) == D.SESSD_E_INVALID
+
+
+def test_sparse2dense_host_side():
+    s = api.Sparse2Dense()
+    blob = s.serialize()
+    assert struct.unpack("<4i", blob) == (176, 200, 2, 64)   # sparse2Dense.cu:288-295
+    assert api.Sparse2Dense.deserialize(blob).serialize() == blob
+    L = api.lib()
+    d = B.dense_desc((176, 0, 2), 64)
+    h = C.c_void_p()
+    assert L.sessd_sparse2dense_create(C.byref(d), C.byref(h)) == D.SESSD_E_INVALID
+
+
+def test_conv_create_validates_before_touching_the_gpu():
+    L = api.lib()
+    h = C.c_void_p()
+    w = np.zeros((27, 4, 16), np.float32)
+    d = D.SubmConv3dDesc()
+    d.in_channel, d.out_channel, d.max_voxels, d.feature_num = 4, 16, 1000, 4
+    for a, v in enumerate((140, 160, 41)):
+        d.out_shape[a] = d.spatial_shape[a] = v
+    d.ksize, d.stride, d.padding, d.dilation = 5, 1, 2, 1      # 125 offsets: beyond the rulebook's 27
+    assert L.sessd_submconv3d_create(C.byref(d), w.ctypes.data_as(C.c_void_p), C.byref(h)) == D.SESSD_E_UNSUPPORTED
+    d.ksize, d.padding, d.stride = 3, 1, 2
+    assert L.sessd_submconv3d_create(C.byref(d), w.ctypes.data_as(C.c_void_p), C.byref(h)) == D.SESSD_E_UNSUPPORTED
+    sd = D.SparseConv3dDesc()
+    sd.in_channel, sd.out_channel, sd.max_voxels = 4, 16, 1000
+    for a in range(3):
+        sd.out_shape[a] = sd.spatial_shape[a] = 10
+        sd.ksize[a], sd.stride[a], sd.padding[a] = 3, 0, 1      # zero stride
+    sd.dilation = 1
+    assert L.sessd_sparseconv3d_create(C.byref(sd), w.ctypes.data_as(C.c_void_p), C.byref(h)) == D.SESSD_E_INVALID
+    assert L.sessd_submconv3d_create(None, None, None) == D.SESSD_E_INVALID
