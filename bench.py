@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Benchmark of the 3-D front end on one MI355X: voxelGenerator -> SpMiddleFHD conv stack -> sparse2Dense.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--points 20000] [--seed 0] [--dtype fp32|fp16]
+
+A "step" is one frame: one pass of the whole path over one seeded synthetic LiDAR frame that is already
+resident in device memory.  The timed region is exactly K pipeline enqueues bracketed by device
+synchronisation.  One JSON line is printed with the frame time, the roofline position of the dominant
+kernel (the 64->64 channel gather-GEMM, timed with HIP events on the pipeline's stream) and the CPU
+baseline (the scalar oracle port, one core, same frame).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "se-ssd-ai-trt_amd"))
+
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+PEAK_FP32_TFLOPS = 157.3    # MI355X dense FP32 (vector and matrix)
+PEAK_FP16_TFLOPS = 2500.0   # MI355X dense FP16 MFMA
+
+
+def layer_work(layer, n_in, n_out, pairs, esize):
+    """Algorithmic work of one conv layer's gather-GEMM launch: flops = 2*P*Cin*Cout; bytes = gathered
+    input rows + output rows written once + rulebook entries read + weights read once."""
+    flops = 2.0 * pairs * layer.cin * layer.cout
+    bytes_ = pairs * layer.cin * esize + n_out * layer.cout * esize + 8.0 * pairs + layer.kvol * layer.cin * layer.cout * esize
+    return flops, bytes_
+
+
+def cpu_baseline(pts, layers, W, max_voxels, budget_s=20.0):
+    """The scalar CPU port (the parity oracle) on the same frame, one thread, a bounded number of frames."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib as O
+    from sessd3d import backbone as B
+    vg = B.voxelgen_desc(max_voxels=max_voxels)
+    dd = B.dense_desc()
+    times = []
+    t_start = time.perf_counter()
+    O.frame(pts, vg, layers, W, dd)          # warm-up (allocates the dense index grids)
+    while len(times) < 5 and (time.perf_counter() - t_start) < budget_s:
+        t0 = time.perf_counter()
+        O.frame(pts, vg, layers, W, dd)
+        times.append((time.perf_counter() - t0) * 1e3)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": round(med, 2), "unit": "ms/frame", "cores": 1, "kind": "port",
+            "sample": "%d frame(s) of the same %d-point frame through oracle_frame (g++ -O2, single thread), median; host has %d logical CPUs"
+                      % (len(times), len(pts), os.cpu_count() or 0)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--points", type=int, default=20000)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--dtype", default="fp32", choices=["fp32", "fp16"])
+    ap.add_argument("--max-voxels", type=int, default=60000)
+    ap.add_argument("--no-graph", action="store_true", help="launch kernels directly instead of replaying a hipGraph")
+    ap.add_argument("--no-share", action="store_true", help="every SubM layer rebuilds its rulebook (as the reference does)")
+    ap.add_argument("--pad-rows", action="store_true", help="write rows >= voxel_num of every tensor (reference behaviour)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--profile-steps", type=int, default=50)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on one GPU (frames are independent; there is no multi-GPU mode); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from sessd3d import api, backbone as B, frames as F
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda:0"
+    layers = B.reference_layers()
+    W = B.random_weights(layers, seed=1, w_std=0.05 if args.dtype == "fp16" else 0.1)
+    pts = F.lidar_frame(args.points, args.seed)
+    max_points = args.points
+    pipe = api.Pipeline(layers, W, max_points, args.max_voxels, feature_dtype=args.dtype,
+                        share_rulebooks=not args.no_share, skip_pad_rows=not args.pad_rows,
+                        use_graph=not args.no_graph)
+    points = torch.as_tensor(pts).to(dev)
+    size = torch.tensor([len(pts)], dtype=torch.int32, device=dev)
+    dense = pipe.new_dense(dev)
+    stream = torch.cuda.Stream()
+
+    with torch.cuda.stream(stream):
+        for _ in range(args.warmup):
+            pipe.enqueue(points, size, dense, stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    with torch.cuda.stream(stream):
+        for _ in range(args.steps):
+            pipe.enqueue(points, size, dense, stream)
+    torch.cuda.synchronize()
+    ms_per_frame = (time.perf_counter() - t0) * 1e3 / args.steps
+    status = pipe.status(stream)
+
+    # per-layer active sites / rulebook pairs (small counting kernels, outside the timed region)
+    n_vox, _ = pipe.layer_stats(-1, stream)
+    stats, n_in = [], n_vox
+    for l, layer in enumerate(layers):
+        n_out, pairs = pipe.layer_stats(l, stream)
+        stats.append((n_in, n_out, pairs))
+        n_in = n_out
+
+    # per-kernel durations: HIP events on the pipeline's stream around every segment, eager launches
+    seg = None
+    with torch.cuda.stream(stream):
+        for _ in range(5):
+            pipe.enqueue_timed(points, size, dense, stream)
+        for _ in range(args.profile_steps):
+            s = np.asarray(pipe.enqueue_timed(points, size, dense, stream), np.float64)
+            seg = s if seg is None else seg + s
+    seg /= args.profile_steps
+    esize = 2 if args.dtype == "fp16" else 4
+    per_layer = []
+    tot_flops = tot_bytes = 0.0
+    for l, layer in enumerate(layers):
+        n_i, n_o, p = stats[l]
+        fl, by = layer_work(layer, n_i, n_o, p, esize)
+        tot_flops += fl
+        tot_bytes += by
+        per_layer.append({"name": layer.name, "n_in": n_i, "n_out": n_o, "pairs": p,
+                          "build_us": round(seg[1 + 2 * l] * 1e3, 2), "gemm_us": round(seg[2 + 2 * l] * 1e3, 2),
+                          "gemm_tflops": round(fl / (seg[2 + 2 * l] * 1e-3) / 1e12, 3) if seg[2 + 2 * l] > 0 else None,
+                          "gemm_gbs": round(by / (seg[2 + 2 * l] * 1e-3) / 1e9, 1) if seg[2 + 2 * l] > 0 else None})
+    # dominant kernel: the gather-GEMM instantiation for 64 -> 64 channels (six launches per frame)
+    dom = [l for l, layer in enumerate(layers) if layer.cin == 64 and layer.cout == 64]
+    dom_flops = sum(layer_work(layers[l], *stats[l], esize)[0] for l in dom) / len(dom)
+    dom_bytes = sum(layer_work(layers[l], *stats[l], esize)[1] for l in dom) / len(dom)
+    dom_ms = sum(seg[2 + 2 * l] for l in dom) / len(dom)
+    peak_tf = PEAK_FP16_TFLOPS if args.dtype == "fp16" else PEAK_FP32_TFLOPS
+    t_mfma = dom_flops / (peak_tf * 1e12)
+    t_hbm = dom_bytes / (PEAK_HBM_GBS * 1e9)
+    if t_mfma >= t_hbm:
+        ach = dom_flops / (dom_ms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": round(ach, 3), "peak": peak_tf, "unit": "TFLOP/s",
+                "frac": round(ach / peak_tf, 4), "traffic": None}
+    else:
+        ach = dom_bytes / (dom_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None}
+    roof.update({"kernel": "gather-GEMM 64->64 (%s)" % args.dtype, "launches_per_frame": len(dom),
+                 "avg_launch_us": round(dom_ms * 1e3, 2), "algorithmic_flops_per_launch": dom_flops,
+                 "algorithmic_bytes_per_launch": dom_bytes})
+    # whole-frame algorithmic traffic: voxelizer + conv layers + sparse2dense (dense tensor written once)
+    c_last, dsz = layers[-1].cout, B.DENSE_SIZE_XYZ
+    frame_bytes = 16.0 * len(pts) + 32.0 * n_vox + tot_bytes + stats[-1][1] * (c_last * esize + 16) + \
+        c_last * dsz[0] * dsz[1] * dsz[2] * esize
+    out = {
+        "metric": "ms/frame voxelize+3D sparse backbone @~17k voxels",
+        "value": round(ms_per_frame, 4), "unit": "ms/frame", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_frame, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16" if args.dtype == "fp16" else "f32", "data": "synthetic",
+        "config": {"workload": "config 3: %d-point seeded synthetic LiDAR frame (seed %d), %d voxels, reference 14-layer "
+                               "SpMiddleFHD backbone (10 SubM + 4 SparseConv, BN folded + ReLU), sparse2Dense to 128x200x176"
+                               % (len(pts), args.seed, n_vox),
+                   "max_voxels": args.max_voxels, "graph": not args.no_graph, "share_rulebooks": not args.no_share,
+                   "pad_rows": args.pad_rows, "n_layers": len(layers)},
+        "roofline": roof,
+        "frame": {"frames_per_s": round(1e3 / ms_per_frame, 1), "algorithmic_gflop": round(tot_flops / 1e9, 3),
+                  "algorithmic_mb": round(frame_bytes / 1e6, 2),
+                  "hbm_roofline_frac": round(frame_bytes / (ms_per_frame * 1e-3) / (PEAK_HBM_GBS * 1e9), 4),
+                  "launches": pipe.num_launches(), "status": status,
+                  "eager_segments_ms": {"voxelize": round(seg[0], 4), "sparse2dense": round(seg[-1], 4),
+                                        "sum": round(float(seg.sum()), 4)}},
+        "layers": per_layer,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(pts, layers, W, args.max_voxels)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

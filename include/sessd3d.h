@@ -74,6 +74,9 @@ enum {
 };
 
 const char* sessd_last_error(void); /* thread-local text of the last failure */
+/* Copy `bytes` from device memory to host memory on `stream` and wait for it: lets a host that has
+ * no HIP binding of its own read back tensors the library owns (see sessd_pipeline_layer_io). */
+int sessd_copy_to_host(void* dst_host, const void* src_device, size_t bytes, sessd_stream_t stream);
 const char* sessd_version(void);
 
 /* ------------------------------------------------------------------------------------------ */
@@ -331,6 +334,16 @@ int sessd_pipeline_enqueue(sessd_pipeline* h, const void* points, const void* po
  * feat: [max_voxels, C]; coors: i32[max_voxels,4]; voxel_num: i32[1]; workspace of that layer. */
 int sessd_pipeline_layer_io(sessd_pipeline* h, int layer, void** feat, void** coors,
                             void** voxel_num, void** workspace, int32_t* channels);
+/* Profiling variant of enqueue: records HIP events on `stream` around the voxelizer, around each
+ * layer's rulebook build and gather-GEMM launch and around sparse2dense, synchronises, and returns
+ * the 2*n_layers+2 segment durations in milliseconds, in that order.  Never uses the graph. */
+int sessd_pipeline_enqueue_timed(sessd_pipeline* h, const void* points, const void* points_size,
+                                 void* dense, sessd_stream_t stream, float* segment_ms,
+                                 int max_segments, int* n_segments);
+/* Active output rows and rulebook pairs of a layer in the last enqueue (layer = -1: voxelizer,
+ * pairs = 0).  Launches small counting kernels and synchronises; for reporting, not the hot path. */
+int sessd_pipeline_layer_stats(sessd_pipeline* h, int layer, sessd_stream_t stream, int64_t* n_out,
+                               int64_t* pairs);
 /* OR of every layer's status word (synchronises the stream) */
 int sessd_pipeline_status(sessd_pipeline* h, sessd_stream_t stream, int32_t* status);
 size_t sessd_pipeline_device_bytes(const sessd_pipeline* h);

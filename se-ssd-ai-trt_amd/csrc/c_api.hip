@@ -25,6 +25,13 @@ extern "C" {
 
 const char* sessd_last_error(void) { return last_error_cstr(); }
 const char* sessd_version(void) { return "sessd3d 0.1 (gfx950)"; }
+int sessd_copy_to_host(void* dst_host, const void* src_device, size_t bytes, sessd_stream_t stream_) {
+    NEED(dst_host && src_device, "null argument");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    SESSD_HIP_TRY(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, stream));
+    SESSD_HIP_TRY(hipStreamSynchronize(stream));
+    return SESSD_OK;
+}
 
 // ------------------------------------------------------------------ voxelgen
 int sessd_voxelgen_create(const sessd_voxelgen_desc* desc, sessd_voxelgen** out) {

@@ -115,7 +115,10 @@ int ConvPluginBase::runGemm(const void* in_feat, void* out_feat, const int32_t* 
     a.shift = epi_.shift_dev;
     a.relu = epi_.relu;
     a.write_pad_rows = (flags_ & SESSD_FLAG_SKIP_PAD_ROWS) ? 0 : 1;
-    return launch_gather_gemm(a, stream);
+    if (ev_gemm_begin_) SESSD_HIP_TRY(hipEventRecord(ev_gemm_begin_, stream));
+    SESSD_TRY(launch_gather_gemm(a, stream));
+    if (ev_gemm_end_) SESSD_HIP_TRY(hipEventRecord(ev_gemm_end_, stream));
+    return SESSD_OK;
 }
 
 int ConvPluginBase::exportRulebook(const int32_t* nbr, const int32_t* num_out, void* scratch,

@@ -159,6 +159,20 @@ size_t export_scratch_bytes(int K, int max_voxels) {
     return align_up(w * sizeof(uint64_t)) + align_up(w * sizeof(uint32_t));
 }
 
+int launch_count_pairs(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, void* scratch,
+                       uint32_t* indice_num, hipStream_t stream) {
+    if (!nbr || !num_out || !scratch || !indice_num) return fail(SESSD_E_INVALID, "count_pairs: null argument");
+    const int wpk = words_per_offset(max_voxels);
+    uint64_t* masks = static_cast<uint64_t*>(scratch);
+    uint32_t* prefix = reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(scratch) +
+                                                   align_up((size_t)K * wpk * sizeof(uint64_t)));
+    hipLaunchKernelGGL(export_masks, dim3(ceil_div(max_voxels, kBlock), K), dim3(kBlock), 0, stream, nbr, num_out,
+                       max_voxels, wpk, masks);
+    hipLaunchKernelGGL(export_scan, dim3(K), dim3(kBlock), 0, stream, masks, wpk, prefix, indice_num);
+    SESSD_HIP_TRY(hipGetLastError());
+    return SESSD_OK;
+}
+
 int launch_export_rulebook(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels,
                            void* scratch, int32_t* indice_pairs, uint32_t* indice_num,
                            hipStream_t stream) {

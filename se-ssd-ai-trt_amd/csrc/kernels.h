@@ -36,4 +36,8 @@ int launch_export_rulebook(const int32_t* nbr, const int32_t* num_out, int K, in
                            void* scratch, int32_t* indice_pairs, uint32_t* indice_num,
                            hipStream_t stream);
 
+// indice_num[k] only (pairs per offset), same scratch as the export
+int launch_count_pairs(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, void* scratch,
+                       uint32_t* indice_num, hipStream_t stream);
+
 }  // namespace sessd

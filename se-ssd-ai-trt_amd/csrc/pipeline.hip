@@ -67,15 +67,24 @@ struct Pipeline {
     void* g_dense = nullptr;
     int graph_nodes = -1;
 
+    // profiling: one event per segment boundary (see sessd_pipeline_enqueue_timed)
+    std::vector<hipEvent_t> events;
+    DeviceBuffer stats;  // u32[32] scratch for per-offset pair counts
+
     ~Pipeline() {
         if (graph_exec) (void)hipGraphExecDestroy(graph_exec);
         if (graph) (void)hipGraphDestroy(graph);
+        for (hipEvent_t e : events) (void)hipEventDestroy(e);
     }
 
     int enqueueDirect(const void* points, const void* points_size, void* dense, hipStream_t stream) {
         const void* vin[2] = {points, points_size};
         void* vout[3] = {vg_voxels.p, vg_coors.p, vg_num.p};
         SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, stream));
+        return enqueueAfterVoxelizer(dense, stream);
+    }
+
+    int enqueueAfterVoxelizer(void* dense, hipStream_t stream) {
         const void* feat = vg_voxels.p;
         const void* coors = vg_coors.p;
         const void* num = vg_num.p;
@@ -365,6 +374,78 @@ int sessd_pipeline_status(sessd_pipeline* h, sessd_stream_t stream_, int32_t* st
     SESSD_TRY(read_status_word(P->s2d_ws.p, 0, stream, &s));
     acc |= s;
     *status = acc;
+    return SESSD_OK;
+}
+
+int sessd_pipeline_enqueue_timed(sessd_pipeline* h, const void* points, const void* points_size, void* dense,
+                                 sessd_stream_t stream_, float* segment_ms, int max_segments, int* n_segments) {
+    if (!h || !points || !points_size || !dense || !segment_ms || !n_segments)
+        return fail(SESSD_E_INVALID, "pipeline_enqueue_timed: null argument");
+    auto* P = reinterpret_cast<Pipeline*>(h);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int L = (int)P->stages.size();
+    const int n_seg = 2 * L + 2;  // voxelizer, {rulebook build, gather-GEMM} per layer, sparse2dense
+    if (max_segments < n_seg) return fail(SESSD_E_INVALID, "pipeline_enqueue_timed: need room for %d segments", n_seg);
+    if (P->events.empty()) {
+        P->events.resize(n_seg + 1);
+        for (auto& e : P->events) SESSD_HIP_TRY(hipEventCreate(&e));
+    }
+    for (int l = 0; l < L; ++l) {
+        ConvPluginBase* b = P->stages[l]->subm ? static_cast<ConvPluginBase*>(P->stages[l]->subm.get())
+                                               : static_cast<ConvPluginBase*>(P->stages[l]->sparse.get());
+        b->ev_gemm_begin_ = P->events[2 + 2 * l];
+        b->ev_gemm_end_ = P->events[3 + 2 * l];
+    }
+    // boundaries: e0 | voxelizer | e1 | build_0 | gb_0 | gemm_0 | ge_0 | build_1 | ... | ge_{L-1} | s2d | e_last
+    // the voxelizer/first-build boundary e1 is recorded by enqueueing the voxelizer separately
+    SESSD_HIP_TRY(hipEventRecord(P->events[0], stream));
+    int rc;
+    {
+        const void* vin[2] = {points, points_size};
+        void* vout[3] = {P->vg_voxels.p, P->vg_coors.p, P->vg_num.p};
+        rc = P->vg->enqueue(P->vg_in, P->vg_out, vin, vout, P->vg_ws.p, stream);
+    }
+    if (rc == SESSD_OK) rc = hipEventRecord(P->events[1], stream) == hipSuccess ? SESSD_OK : SESSD_E_HIP;
+    if (rc == SESSD_OK) rc = P->enqueueAfterVoxelizer(dense, stream);
+    if (rc == SESSD_OK) rc = hipEventRecord(P->events[n_seg], stream) == hipSuccess ? SESSD_OK : SESSD_E_HIP;
+    for (int l = 0; l < L; ++l) {
+        ConvPluginBase* b = P->stages[l]->subm ? static_cast<ConvPluginBase*>(P->stages[l]->subm.get())
+                                               : static_cast<ConvPluginBase*>(P->stages[l]->sparse.get());
+        b->ev_gemm_begin_ = b->ev_gemm_end_ = nullptr;
+    }
+    SESSD_TRY(rc);
+    SESSD_HIP_TRY(hipStreamSynchronize(stream));
+    for (int i = 0; i < n_seg; ++i)
+        SESSD_HIP_TRY(hipEventElapsedTime(&segment_ms[i], P->events[i], P->events[i + 1]));
+    *n_segments = n_seg;
+    return SESSD_OK;
+}
+
+int sessd_pipeline_layer_stats(sessd_pipeline* h, int layer, sessd_stream_t stream_, int64_t* n_out,
+                               int64_t* pairs) {
+    if (!h || !n_out || !pairs) return fail(SESSD_E_INVALID, "pipeline_layer_stats: null argument");
+    auto* P = reinterpret_cast<Pipeline*>(h);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (layer < -1 || layer >= (int)P->stages.size()) return fail(SESSD_E_INVALID, "pipeline_layer_stats: no layer %d", layer);
+    void* num = nullptr;
+    void* ws = nullptr;
+    SESSD_TRY(sessd_pipeline_layer_io(h, layer, nullptr, nullptr, &num, &ws, nullptr));
+    int32_t n = 0;
+    SESSD_HIP_TRY(hipMemcpyAsync(&n, num, sizeof(n), hipMemcpyDeviceToHost, stream));
+    SESSD_HIP_TRY(hipStreamSynchronize(stream));
+    *n_out = n;
+    *pairs = 0;
+    if (layer < 0) return SESSD_OK;
+    if (!P->stats.p) SESSD_TRY(P->stats.alloc(32 * sizeof(uint32_t)));
+    ConvStage& st = *P->stages[layer];
+    uint32_t* dev_num = static_cast<uint32_t*>(P->stats.p);
+    const int K = st.spec.ksize[0] * st.spec.ksize[1] * st.spec.ksize[2];
+    if (st.subm) SESSD_TRY(st.subm->countPairs(ws, dev_num, stream));
+    else SESSD_TRY(st.sparse->countPairs(ws, dev_num, stream));
+    uint32_t host[32] = {0};
+    SESSD_HIP_TRY(hipMemcpyAsync(host, dev_num, K * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    SESSD_HIP_TRY(hipStreamSynchronize(stream));
+    for (int k = 0; k < K; ++k) *pairs += host[k];
     return SESSD_OK;
 }
 

@@ -79,6 +79,8 @@ class ConvPluginBase {
     Epilogue epi_;
     int in_type_ = SESSD_FLOAT, out_type_ = SESSD_FLOAT;
     int flags_ = 0;
+    // when set, recorded on the stream right before / after the gather-GEMM launch (profiling)
+    hipEvent_t ev_gemm_begin_ = nullptr, ev_gemm_end_ = nullptr;
 
   protected:
     // gather-GEMM over the neighbour table nbr[K][max_voxels] (device), rows < *num_out
@@ -111,6 +113,7 @@ class SubmConv3dLayerPlugin : public ConvPluginBase {
                       const void* rulebook_workspace, hipStream_t stream);
     int exportRulebook(const void* workspace, int32_t* indice_pairs, uint32_t* indice_num,
                        hipStream_t stream) const;
+    int countPairs(const void* workspace, uint32_t* indice_num, hipStream_t stream) const;
     size_t getSerializationSize() const;
     void serialize(void* buffer) const;
     size_t statusOffset() const;
@@ -141,6 +144,7 @@ class SparseConv3dLayerPlugin : public ConvPluginBase {
                 hipStream_t stream);
     int exportRulebook(const void* workspace, int32_t* indice_pairs, uint32_t* indice_num,
                        hipStream_t stream) const;
+    int countPairs(const void* workspace, uint32_t* indice_num, hipStream_t stream) const;
     size_t getSerializationSize() const;
     void serialize(void* buffer) const;
     size_t statusOffset() const;

@@ -386,4 +386,10 @@ int SparseConv3dLayerPlugin::exportRulebook(const void* workspace, int32_t* indi
     return ConvPluginBase::exportRulebook(L.nbr, L.meta + 1, L.export_scratch, indice_pairs, indice_num, stream);
 }
 
+int SparseConv3dLayerPlugin::countPairs(const void* workspace, uint32_t* indice_num, hipStream_t stream) const {
+    if (!workspace) return fail(SESSD_E_INVALID, "sparseconv3d.count_pairs: workspace is null");
+    const Layout L = carve(const_cast<void*>(workspace));
+    return launch_count_pairs(L.nbr, L.meta + 1, kernel_volume_, max_voxels_, L.export_scratch, indice_num, stream);
+}
+
 }  // namespace sessd

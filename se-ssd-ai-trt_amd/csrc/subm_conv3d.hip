@@ -261,4 +261,10 @@ int SubmConv3dLayerPlugin::exportRulebook(const void* workspace, int32_t* indice
     return ConvPluginBase::exportRulebook(L.nbr, L.meta + 1, L.export_scratch, indice_pairs, indice_num, stream);
 }
 
+int SubmConv3dLayerPlugin::countPairs(const void* workspace, uint32_t* indice_num, hipStream_t stream) const {
+    if (!workspace) return fail(SESSD_E_INVALID, "submconv3d.count_pairs: workspace is null");
+    const Layout L = carve(const_cast<void*>(workspace));
+    return launch_count_pairs(L.nbr, L.meta + 1, kernel_volume_, max_voxels_, L.export_scratch, indice_num, stream);
+}
+
 }  // namespace sessd

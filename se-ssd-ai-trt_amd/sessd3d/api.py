@@ -38,6 +38,12 @@ def lib():
         return _lib
     if not os.path.exists(LIB_PATH):
         raise SessdError("libsessd3d.so is not built: run `python se-ssd-ai-trt_amd/build.py` (%s)" % LIB_PATH)
+    # torch bundles its own HIP runtime under the same soname as the system one.  A process must hold
+    # exactly one: import torch first so that the library binds to the runtime torch's tensors live in.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = C.CDLL(LIB_PATH)
     vp, sz, i32 = C.c_void_p, C.c_size_t, C.c_int32
     TD = C.POINTER(D.TensorDesc)
@@ -73,11 +79,14 @@ def lib():
     L.sessd_pipeline_enqueue.argtypes = [vp, vp, vp, vp, vp]
     L.sessd_pipeline_layer_io.argtypes = [vp, C.c_int, VPP, VPP, VPP, VPP, C.POINTER(i32)]
     L.sessd_pipeline_status.argtypes = [vp, vp, C.POINTER(i32)]
+    L.sessd_pipeline_enqueue_timed.argtypes = [vp, vp, vp, vp, vp, C.POINTER(C.c_float), C.c_int, C.POINTER(C.c_int)]
+    L.sessd_pipeline_layer_stats.argtypes = [vp, C.c_int, vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
     L.sessd_pipeline_device_bytes.restype = sz
     L.sessd_pipeline_device_bytes.argtypes = [vp]
     L.sessd_pipeline_num_launches.argtypes = [vp]
     L.sessd_pipeline_destroy.argtypes = [vp]
     L.sessd_pipeline_destroy.restype = None
+    L.sessd_copy_to_host.argtypes = [vp, vp, sz, vp]
     _lib = L
     return L
 
@@ -405,6 +414,21 @@ class Pipeline:
         check(lib().sessd_pipeline_status(self.h, _stream_ptr(stream), C.byref(s)))
         return s.value
 
+    def enqueue_timed(self, points, points_size, dense, stream=None):
+        """-> list of segment durations in ms: [voxelizer, (build, gemm) per layer ..., sparse2dense]"""
+        nseg = 2 * len(self.layers) + 2
+        ms = (C.c_float * nseg)()
+        got = C.c_int(0)
+        check(lib().sessd_pipeline_enqueue_timed(self.h, _ptr(points), _ptr(points_size), _ptr(dense),
+                                                 _stream_ptr(stream), ms, nseg, C.byref(got)))
+        return list(ms)[:got.value]
+
+    def layer_stats(self, layer, stream=None):
+        """-> (active output rows, rulebook pairs) of `layer` in the last enqueue"""
+        n, p = C.c_int64(0), C.c_int64(0)
+        check(lib().sessd_pipeline_layer_stats(self.h, layer, _stream_ptr(stream), C.byref(n), C.byref(p)))
+        return n.value, p.value
+
     def device_bytes(self):
         return lib().sessd_pipeline_device_bytes(self.h)
 
@@ -423,15 +447,6 @@ class Pipeline:
             pass
 
 
-_hip = None
-
-
 def _hip_d2h(dst_np, src_ptr):
-    """hipMemcpy device->host into a numpy array (for pointers owned by the library)."""
-    global _hip
-    if _hip is None:
-        _hip = C.CDLL("libamdhip64.so")
-        _hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
-    rc = _hip.hipMemcpy(dst_np.ctypes.data_as(C.c_void_p), C.c_void_p(src_ptr), dst_np.nbytes, 2)
-    if rc != 0:
-        raise SessdError("hipMemcpy D2H failed: %d" % rc)
+    """Synchronous device->host copy into a numpy array (for pointers owned by the library)."""
+    check(lib().sessd_copy_to_host(dst_np.ctypes.data_as(C.c_void_p), C.c_void_p(src_ptr), dst_np.nbytes, None))

@@ -22,16 +22,34 @@ def run_pipeline(pts, layers, W, max_points, max_voxels, **kw):
     return pipe, dense, (p, n, stream)
 
 
-def compare_with_oracle(pipe, dense, pts, layers, W, max_voxels, rtol):
+# End to end the FP32 rounding differences of 14 stacked layers compound (each layer's error is amplified
+# by the next layer's weights and by cancellation), so the whole-frame comparison uses 1e-3; the 1e-4
+# bound is checked layer by layer, each layer of the oracle being fed the GPU's own input rows.
+RTOL_END_TO_END = 1e-3
+
+
+def compare_with_oracle(pipe, dense, pts, layers, W, max_voxels, rtol_layer, rtol_frame=RTOL_END_TO_END):
     ref = O.frame(pts, B.voxelgen_desc(max_voxels=max_voxels), layers, W, B.dense_desc())
-    counts = [pipe.read_layer(l)[2] for l in range(-1, len(layers))]
-    assert counts == ref["counts"].tolist()
-    feat, coors, n = pipe.read_layer(len(layers) - 1)
-    assert np.array_equal(coors, ref["coors"])                       # same numbering, row by row
+    feat, coors, n = pipe.read_layer(-1)
+    assert n == ref["counts"][0]
+    for l, layer in enumerate(layers):
+        fbuf = np.zeros((max_voxels, layer.cin), np.float32)
+        fbuf[:n] = feat
+        cbuf = np.zeros((max_voxels, 4), np.int32)
+        cbuf[:n] = coors
+        o_out, o_coors, o_n, _, _ = O.conv_layer(fbuf, cbuf, n, layer, W.w[l], W.scale[l], W.shift[l], max_voxels)
+        feat, g_coors, g_n = pipe.read_layer(l)
+        assert g_n == o_n == ref["counts"][l + 1], layer.name
+        assert np.array_equal(g_coors, o_coors[:o_n]), layer.name          # same numbering, row by row
+        assert_features_close(feat, o_out[:o_n], rtol_layer, layer.name)
+        coors, n = g_coors, g_n
+    assert np.array_equal(coors, ref["coors"])
     a, b = canonical(coors, n, feat), canonical(ref["coors"], n, ref["feat"])
     assert np.array_equal(a[0], b[0])
-    assert_features_close(a[1], b[1], rtol, "last layer features")
-    assert_features_close(to_np(dense).astype(np.float32), ref["dense"], rtol, "dense BEV tensor")
+    assert_features_close(a[1], b[1], rtol_frame, "last layer features (end to end)")
+    assert_features_close(to_np(dense).astype(np.float32), ref["dense"], rtol_frame, "dense BEV tensor (end to end)")
+    # the dense tensor is an exact scatter of the last layer's rows
+    assert np.array_equal(to_np(dense).astype(np.float32), O.sparse2dense(feat, coors, n, B.DENSE_SIZE_XYZ))
     assert pipe.status() == ref["status"]
     return ref
 
@@ -77,7 +95,7 @@ def test_full_backbone_config3_frame_and_graph_replay():
         gpipe.enqueue(p, n, gd, stream)
     stream.synchronize()
     ref2 = O.frame(pts2, B.voxelgen_desc(max_voxels=60000), layers, W, B.dense_desc())
-    assert_features_close(to_np(gd), ref2["dense"], RTOL_FP32, "graph replay on a new frame")
+    assert_features_close(to_np(gd), ref2["dense"], RTOL_END_TO_END, "graph replay on a new frame")
 
 
 def test_properties_at_full_size():
