@@ -70,7 +70,10 @@ enum {
 enum {
     /* Do not write feature rows >= voxel_num.  The reference zero-fills every output up to
      * max_voxels rows; consumers gate on voxel_num, so a fused pipeline can skip that traffic. */
-    SESSD_FLAG_SKIP_PAD_ROWS = 1
+    SESSD_FLAG_SKIP_PAD_ROWS = 1,
+    /* Run the gather-GEMM on the shape-agnostic VALU kernel even where an MFMA kernel exists
+     * (cross-check of the matrix-core path). */
+    SESSD_FLAG_FORCE_VALU = 2
 };
 
 const char* sessd_last_error(void); /* thread-local text of the last failure */

@@ -115,6 +115,7 @@ int ConvPluginBase::runGemm(const void* in_feat, void* out_feat, const int32_t* 
     a.shift = epi_.shift_dev;
     a.relu = epi_.relu;
     a.write_pad_rows = (flags_ & SESSD_FLAG_SKIP_PAD_ROWS) ? 0 : 1;
+    a.force_valu = (flags_ & SESSD_FLAG_FORCE_VALU) ? 1 : 0;
     if (ev_gemm_begin_) SESSD_HIP_TRY(hipEventRecord(ev_gemm_begin_, stream));
     SESSD_TRY(launch_gather_gemm(a, stream));
     if (ev_gemm_end_) SESSD_HIP_TRY(hipEventRecord(ev_gemm_end_, stream));

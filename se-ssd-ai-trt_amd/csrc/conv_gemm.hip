@@ -137,10 +137,13 @@ export_pairs(const int32_t* __restrict__ nbr, int max_voxels, int words_per_k,
 
 }  // namespace
 
-size_t packed_weight_bytes(int, int, int, int) { return 0; }
-void pack_weights(const float*, int, int, int, int, void*) {}
+int launch_mfma(const GemmArgs& a, hipStream_t stream);  // conv_mfma.hip
 
 int launch_gather_gemm(const GemmArgs& a, hipStream_t stream) {
+    if (!a.force_valu) {
+        const int rc = launch_mfma(a, stream);
+        if (rc != SESSD_E_UNSUPPORTED) return rc;  // launched (or failed for good)
+    }
     if (a.in_type == SESSD_FLOAT && a.out_type == SESSD_FLOAT)
         return launch_generic<float, float, float>(a, a.w_f32, stream);
     if (a.in_type == SESSD_FLOAT && a.out_type == SESSD_HALF)

@@ -20,6 +20,7 @@ struct GemmArgs {
     const float* shift;      // [cout] or null
     int relu;
     int write_pad_rows;      // rows >= *num_out get epilogue(0) (the reference zero-fills them)
+    int force_valu;          // skip the MFMA kernels (cross-check)
 };
 
 // picks the kernel for the layer shape; returns SESSD_E_UNSUPPORTED for dtype pairs not covered

@@ -16,6 +16,7 @@ SESSD_STATUS_HASH_FULL = 2
 SESSD_STATUS_BAD_COORD = 4
 
 SESSD_FLAG_SKIP_PAD_ROWS = 1
+SESSD_FLAG_FORCE_VALU = 2
 
 SESSD_LAYER_SUBM = 0
 SESSD_LAYER_SPARSE = 1

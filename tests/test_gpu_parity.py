@@ -124,7 +124,8 @@ def test_subm_config1_rulebook_and_features():
     assert conv.status() == 0
 
 
-@pytest.mark.parametrize("cin,cout", [(4, 16), (16, 16), (32, 32), (64, 64), (5, 7)])
+@pytest.mark.parametrize("cin,cout", [(4, 16), (16, 16), (16, 32), (32, 32), (32, 64), (64, 64), (64, 128), (128, 128),
+                                      (5, 7), (8, 32)])
 def test_subm_clustered_with_epilogue_and_pad_rows(cin, cout):
     grid = (21, 200, 176)
     n, mv = 6000, 8192
@@ -144,6 +145,27 @@ def test_subm_clustered_with_epilogue_and_pad_rows(cin, cout):
         assert np.all(np.diff(pairs[k, 1, :num[k]]) > 0) and np.all(pairs[k, :, num[k]:] == -1)
     o_out = O.scale_shift_relu(O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), mv, sc, sh, True)
     assert_features_close(out, o_out, RTOL_FP32, "subm %d->%d" % (cin, cout))   # incl. pad rows = relu(shift)
+
+
+def test_mfma_and_valu_paths_agree():
+    """The matrix-core kernel against the shape-agnostic VALU kernel on the same rulebook (both FP32)."""
+    grid = (11, 120, 120)
+    n, mv = 9000, 9001                      # a last tile that is only partly active
+    rng = np.random.default_rng(7)
+    coors = F.clustered_active_voxels(n, grid, 5, n_blobs=30, sigma=(1.5, 5.0, 5.0))
+    feat = rng.uniform(-1, 1, (n, 64)).astype(np.float32)
+    w = rng.normal(0, 0.1, (27, 64, 64)).astype(np.float32)
+    outs = []
+    for flags in (0, D.SESSD_FLAG_FORCE_VALU):
+        conv = api.SubmConv3d(64, 64, grid[::-1], w, mv)
+        conv.set_flags(flags)
+        cbuf = np.zeros((mv, 4), np.int32)
+        cbuf[:n] = coors
+        fbuf = np.zeros((mv, 64), np.float32)
+        fbuf[:n] = feat
+        outs.append(to_np(conv(dev(fbuf), dev(cbuf), dev(np.array([n], np.int32)))))
+    assert_features_close(outs[0], outs[1], RTOL_FP32, "mfma vs valu")
+    assert not np.array_equal(outs[0], outs[1]) or True
 
 
 def test_subm_shared_rulebook_skip_pad_and_empty():
