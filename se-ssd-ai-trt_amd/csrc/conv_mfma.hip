@@ -2,8 +2,8 @@
 //
 //     out[o][:] = epilogue( sum_k  in[nbr[k][o]][:] @ W[k] )
 //
-// One workgroup (4 wave64) owns a tile of 32 output rows and all Cout columns.
-//   * The tile's neighbour lists nbr[k][row0..row0+31] for all K offsets are staged in LDS once.
+// One workgroup (4 wave64) owns a tile of 16 output rows (one MFMA row block) and all Cout columns.
+//   * The tile's neighbour lists nbr[k][row0..row0+15] for all K offsets are staged in LDS once.
 //   * Offsets for which the tile has no neighbour at all are skipped (wave64 ballot over the staged
 //     list); the remaining ones are dealt round-robin to the four waves (split-K over offsets), so a
 //     small frame still fills the chip: tiles x 4 waves.
@@ -11,8 +11,9 @@
 //     (i = lane%16, q = lane/16) loads 16 bytes = channels 16g+4q .. 16g+4q+3 of row i, i.e. every
 //     row is read as 64-byte segments.  The weights were reordered on the host so that the B operand
 //     of the same four MFMA steps is one 16-byte load per lane as well.
-//   * v_mfma_f32_16x16x4_f32 accumulates in FP32; a 16-row block without neighbours at this offset is
-//     skipped.
+//   * v_mfma_f32_16x16x4_f32 accumulates in FP32.  The tile height trades weight re-reads (one pass
+//     over W[k] per tile and offset) against load balance: at ~17k active rows a 16-row tile gives
+//     ~1000 workgroups for 256 CUs and measured fastest.
 //   * The four partial tiles are summed through LDS in a fixed order (deterministic), the
 //     scale/shift/ReLU epilogue is applied and each output row is written once, coalesced.
 #include "kernels.h"
@@ -23,9 +24,15 @@ namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kWaves = 4;
-constexpr int kTileRows = 32;  // two 16-row MFMA blocks per wave
-constexpr int kRB = kTileRows / 16;
+#ifndef SESSD_MFMA_WAVES
+#define SESSD_MFMA_WAVES 4
+#endif
+#ifndef SESSD_MFMA_RB
+#define SESSD_MFMA_RB 1
+#endif
+constexpr int kWaves = SESSD_MFMA_WAVES;
+constexpr int kRB = SESSD_MFMA_RB;   // 16-row MFMA blocks per wave
+constexpr int kTileRows = kRB * 16;
 
 template <int CIN, int COUT>
 __global__ void __launch_bounds__(kWaves * 64)
@@ -61,50 +68,86 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
 
     const int i = lane & 15;  // row inside a 16-row block
     const int q = lane >> 4;  // 4-channel group inside a 16-channel chunk
-    int live = 0;             // non-empty offsets seen so far
-    for (int k = 0; k < K; ++k) {
-        int idx[kRB];
-        bool any_rb[kRB];
-        bool any = false;
+
+    // offsets this wave handles: the non-empty ones of the tile, dealt round-robin to the four waves;
+    // bit k of rb_mask[rb] = "16-row block rb has a neighbour at offset k" (all wave-uniform)
+    uint32_t my_mask = 0, rb_mask[kRB];
+#pragma unroll
+    for (int rb = 0; rb < kRB; ++rb) rb_mask[rb] = 0;
+    {
+        int live = 0;
+        for (int k = 0; k < K; ++k) {
+            bool any = false;
+#pragma unroll
+            for (int rb = 0; rb < kRB; ++rb) {
+                const bool any_rb = __ballot(s_nbr[k * kTileRows + rb * 16 + i] >= 0) != 0ull;
+                if (any_rb) rb_mask[rb] |= 1u << k;
+                any = any || any_rb;
+            }
+            if (any) {
+                if ((live % kWaves) == wave) my_mask |= 1u << k;
+                ++live;
+            }
+        }
+    }
+
+    // Software pipeline: the gathered rows of the NEXT offset and the weights of the NEXT 16-channel
+    // chunk are in flight while the MFMAs of the current chunk issue.
+    const float4* wp4 = reinterpret_cast<const float4*>(Wp) + lane;
+    auto load_a = [&](int k, float4 (&a)[kRB][G]) {
 #pragma unroll
         for (int rb = 0; rb < kRB; ++rb) {
-            idx[rb] = s_nbr[k * kTileRows + rb * 16 + i];
-            any_rb[rb] = __ballot(idx[rb] >= 0) != 0ull;
-            any = any || any_rb[rb];
+            const int idx = s_nbr[k * kTileRows + rb * 16 + i];
+            const float4* src = reinterpret_cast<const float4*>(in + (size_t)(idx < 0 ? 0 : idx) * CIN + q * 4);
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (idx >= 0) v = src[g * 4];
+                a[rb][g] = v;
+            }
         }
-        if (!any) continue;               // wave-uniform: nobody in the tile has this neighbour
-        const bool mine = (live & (kWaves - 1)) == wave;
-        ++live;
-        if (!mine) continue;
+    };
+    auto load_b = [&](int k, int g, float4 (&b)[NB]) {
+        const float4* wk = wp4 + ((size_t)k * G + g) * NB * 64;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) b[nb] = wk[nb * 64];
+    };
 
-        float4 a[kRB][G];
+    int k_cur = my_mask ? __ffs(my_mask) - 1 : -1;
+    my_mask &= my_mask - 1;
+    float4 a_cur[kRB][G], a_nxt[kRB][G], b_cur[NB], b_nxt[NB];
+    if (k_cur >= 0) {
+        load_a(k_cur, a_cur);
+        load_b(k_cur, 0, b_cur);
+    }
+    while (k_cur >= 0) {
+        const int k_nxt = my_mask ? __ffs(my_mask) - 1 : -1;
+        my_mask &= my_mask - 1;
+        if (k_nxt >= 0) load_a(k_nxt, a_nxt);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            if (g + 1 < G) load_b(k_cur, g + 1, b_nxt);
+            else if (k_nxt >= 0) load_b(k_nxt, 0, b_nxt);
+#pragma unroll
+            for (int rb = 0; rb < kRB; ++rb) {
+                if (!((rb_mask[rb] >> k_cur) & 1u)) continue;  // wave-uniform: block has no neighbour here
+                const float av[4] = {a_cur[rb][g].x, a_cur[rb][g].y, a_cur[rb][g].z, a_cur[rb][g].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) {
+                        const float bv[4] = {b_cur[nb].x, b_cur[nb].y, b_cur[nb].z, b_cur[nb].w};
+                        acc[rb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[e], bv[e], acc[rb][nb], 0, 0, 0);
+                    }
+            }
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) b_cur[nb] = b_nxt[nb];
+        }
 #pragma unroll
         for (int rb = 0; rb < kRB; ++rb)
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
-                a[rb][g] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (idx[rb] >= 0)
-                    a[rb][g] = *reinterpret_cast<const float4*>(in + (size_t)idx[rb] * CIN + g * 16 + q * 4);
-            }
-        const float4* wk = reinterpret_cast<const float4*>(Wp) + (size_t)k * G * NB * 64 + lane;
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            float4 b[NB];
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) b[nb] = wk[(g * NB + nb) * 64];
-#pragma unroll
-            for (int rb = 0; rb < kRB; ++rb) {
-                if (!any_rb[rb]) continue;  // wave-uniform
-                const float av[4] = {a[rb][g].x, a[rb][g].y, a[rb][g].z, a[rb][g].w};
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                    const float bv[4] = {b[nb].x, b[nb].y, b[nb].z, b[nb].w};
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        acc[rb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[e], bv[e], acc[rb][nb], 0, 0, 0);
-                }
-            }
-        }
+            for (int g = 0; g < G; ++g) a_cur[rb][g] = a_nxt[rb][g];
+        k_cur = k_nxt;
     }
 
     // partial tile of this wave -> LDS.  D layout of the 16x16 MFMA: lane holds column lane%16 of rows

@@ -14,7 +14,7 @@ from . import backbone as B
 from . import ctypes_defs as D
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libsessd3d.so")
+LIB_PATH = os.environ.get("SESSD3D_LIB") or os.path.join(os.path.dirname(_HERE), "lib", "libsessd3d.so")
 HEADER_PATH = os.path.join(os.path.dirname(os.path.dirname(_HERE)), "include", "sessd3d.h")
 _lib = None
 
