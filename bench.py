@@ -31,6 +31,21 @@ def layer_work(layer, n_in, n_out, pairs, esize):
     return flops, bytes_
 
 
+def profiled_traffic(kernel, dtype):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 summary (FETCH_SIZE and WRITE_SIZE
+    runs, scaled by a copy kernel of known size), or None when no summary covers it."""
+    path = os.path.join(ROOT, "profiles", "frame_pipeline_config3_%s.md" % dtype)
+    try:
+        with open(path) as f:
+            for line in f:
+                cells = [c.strip() for c in line.split("|")]
+                if len(cells) >= 8 and cells[1] == kernel and cells[2].isdigit():
+                    return (float(cells[5]) + float(cells[6])) * 1e6
+    except (OSError, ValueError):
+        pass
+    return None
+
+
 def cpu_baseline(pts, layers, W, max_voxels, budget_s=20.0):
     """The scalar CPU port (the parity oracle) on the same frame, one thread, a bounded number of frames."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
@@ -66,6 +81,9 @@ def main():
     ap.add_argument("--pad-rows", action="store_true", help="write rows >= voxel_num of every tensor (reference behaviour)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--profile-steps", type=int, default=50)
+    ap.add_argument("--calibrate-mb", type=int, default=0,
+                    help="after the timed region run a device-to-device copy of this many MiB three times: a kernel "
+                         "of known traffic against which rocprofv3's FETCH_SIZE / WRITE_SIZE counters are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on one GPU (frames are independent; there is no multi-GPU mode); use --gpus 1",
@@ -111,14 +129,21 @@ def main():
         n_in = n_out
 
     # per-kernel durations: HIP events on the pipeline's stream around every segment, eager launches
-    seg = None
+    # (an event pair that brackets nothing still reads a few microseconds: that empty-segment time is
+    # measured in the same pass and subtracted from every segment)
+    seg, empty = None, 0.0
     with torch.cuda.stream(stream):
         for _ in range(5):
             pipe.enqueue_timed(points, size, dense, stream)
         for _ in range(args.profile_steps):
-            s = np.asarray(pipe.enqueue_timed(points, size, dense, stream), np.float64)
+            s, e = pipe.enqueue_timed(points, size, dense, stream)
+            s = np.asarray(s, np.float64)
             seg = s if seg is None else seg + s
+            empty += e
     seg /= args.profile_steps
+    empty /= args.profile_steps
+    raw_sum = float(seg.sum())
+    seg = np.maximum(seg - empty, 0.0)
     esize = 2 if args.dtype == "fp16" else 4
     per_layer = []
     tot_flops = tot_bytes = 0.0
@@ -147,6 +172,7 @@ def main():
         ach = dom_bytes / (dom_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None}
+    roof["traffic"] = profiled_traffic("conv_mfma_%s<64, 64>" % ("f16" if args.dtype == "fp16" else "f32"), args.dtype)
     roof.update({"kernel": "gather-GEMM 64->64 (%s)" % args.dtype, "launches_per_frame": len(dom),
                  "avg_launch_us": round(dom_ms * 1e3, 2), "algorithmic_flops_per_launch": dom_flops,
                  "algorithmic_bytes_per_launch": dom_bytes})
@@ -170,9 +196,17 @@ def main():
                   "hbm_roofline_frac": round(frame_bytes / (ms_per_frame * 1e-3) / (PEAK_HBM_GBS * 1e9), 4),
                   "launches": pipe.num_launches(), "status": status,
                   "eager_segments_ms": {"voxelize": round(seg[0], 4), "sparse2dense": round(seg[-1], 4),
-                                        "sum": round(float(seg.sum()), 4)}},
+                                        "sum_raw": round(raw_sum, 4), "empty_segment": round(empty, 5)}},
         "layers": per_layer,
     }
+    if args.calibrate_mb > 0:
+        src = torch.full((args.calibrate_mb * (1 << 20) // 4,), 1.5, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        out["calibration"] = {"copy_mib": args.calibrate_mb, "repeats": 3}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(pts, layers, W, args.max_voxels)
     print(json.dumps(out))

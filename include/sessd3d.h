@@ -339,7 +339,9 @@ int sessd_pipeline_layer_io(sessd_pipeline* h, int layer, void** feat, void** co
                             void** voxel_num, void** workspace, int32_t* channels);
 /* Profiling variant of enqueue: records HIP events on `stream` around the voxelizer, around each
  * layer's rulebook build and gather-GEMM launch and around sparse2dense, synchronises, and returns
- * the 2*n_layers+2 segment durations in milliseconds, in that order.  Never uses the graph. */
+ * the 2*n_layers+2 segment durations in milliseconds, in that order.  When max_segments leaves room
+ * for one more value, segment_ms[2*n_layers+2] receives the time between two events recorded back to
+ * back (what the timer itself adds to every segment).  Never uses the graph. */
 int sessd_pipeline_enqueue_timed(sessd_pipeline* h, const void* points, const void* points_size,
                                  void* dense, sessd_stream_t stream, float* segment_ms,
                                  int max_segments, int* n_segments);

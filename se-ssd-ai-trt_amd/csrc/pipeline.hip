@@ -387,7 +387,7 @@ int sessd_pipeline_enqueue_timed(sessd_pipeline* h, const void* points, const vo
     const int n_seg = 2 * L + 2;  // voxelizer, {rulebook build, gather-GEMM} per layer, sparse2dense
     if (max_segments < n_seg) return fail(SESSD_E_INVALID, "pipeline_enqueue_timed: need room for %d segments", n_seg);
     if (P->events.empty()) {
-        P->events.resize(n_seg + 1);
+        P->events.resize(n_seg + 3);  // + two back-to-back events that bracket nothing (timer overhead)
         for (auto& e : P->events) SESSD_HIP_TRY(hipEventCreate(&e));
     }
     for (int l = 0; l < L; ++l) {
@@ -398,6 +398,8 @@ int sessd_pipeline_enqueue_timed(sessd_pipeline* h, const void* points, const vo
     }
     // boundaries: e0 | voxelizer | e1 | build_0 | gb_0 | gemm_0 | ge_0 | build_1 | ... | ge_{L-1} | s2d | e_last
     // the voxelizer/first-build boundary e1 is recorded by enqueueing the voxelizer separately
+    SESSD_HIP_TRY(hipEventRecord(P->events[n_seg + 1], stream));
+    SESSD_HIP_TRY(hipEventRecord(P->events[n_seg + 2], stream));
     SESSD_HIP_TRY(hipEventRecord(P->events[0], stream));
     int rc;
     {
@@ -417,6 +419,8 @@ int sessd_pipeline_enqueue_timed(sessd_pipeline* h, const void* points, const vo
     SESSD_HIP_TRY(hipStreamSynchronize(stream));
     for (int i = 0; i < n_seg; ++i)
         SESSD_HIP_TRY(hipEventElapsedTime(&segment_ms[i], P->events[i], P->events[i + 1]));
+    if (max_segments > n_seg)  // optional extra slot: what an empty segment measures on this stream
+        SESSD_HIP_TRY(hipEventElapsedTime(&segment_ms[n_seg], P->events[n_seg + 1], P->events[n_seg + 2]));
     *n_segments = n_seg;
     return SESSD_OK;
 }

@@ -415,13 +415,14 @@ class Pipeline:
         return s.value
 
     def enqueue_timed(self, points, points_size, dense, stream=None):
-        """-> list of segment durations in ms: [voxelizer, (build, gemm) per layer ..., sparse2dense]"""
+        """-> (segment durations in ms: [voxelizer, (build, gemm) per layer ..., sparse2dense],
+              duration of an empty segment = what the event pair itself measures)"""
         nseg = 2 * len(self.layers) + 2
-        ms = (C.c_float * nseg)()
+        ms = (C.c_float * (nseg + 1))()
         got = C.c_int(0)
         check(lib().sessd_pipeline_enqueue_timed(self.h, _ptr(points), _ptr(points_size), _ptr(dense),
-                                                 _stream_ptr(stream), ms, nseg, C.byref(got)))
-        return list(ms)[:got.value]
+                                                 _stream_ptr(stream), ms, nseg + 1, C.byref(got)))
+        return list(ms)[:got.value], float(ms[got.value])
 
     def layer_stats(self, layer, stream=None):
         """-> (active output rows, rulebook pairs) of `layer` in the last enqueue"""
