@@ -2,20 +2,25 @@
 //
 //     out[o][:] = epilogue( sum_k  in[nbr[k][o]][:] @ W[k] )
 //
-// One workgroup (4 wave64) owns a tile of 16 output rows (one MFMA row block) and all Cout columns.
-//   * The tile's neighbour lists nbr[k][row0..row0+15] for all K offsets are staged in LDS once.
-//   * Offsets for which the tile has no neighbour at all are skipped (wave64 ballot over the staged
-//     list); the remaining ones are dealt round-robin to the four waves (split-K over offsets), so a
-//     small frame still fills the chip: tiles x 4 waves.
-//   * A wave gathers the input rows of an offset straight into MFMA A-operand registers: lane
-//     (i = lane%16, q = lane/16) loads 16 bytes = channels 16g+4q .. 16g+4q+3 of row i, i.e. every
-//     row is read as 64-byte segments.  The weights were reordered on the host so that the B operand
-//     of the same four MFMA steps is one 16-byte load per lane as well.
-//   * v_mfma_f32_16x16x4_f32 accumulates in FP32.  The tile height trades weight re-reads (one pass
-//     over W[k] per tile and offset) against load balance: at ~17k active rows a 16-row tile gives
-//     ~1000 workgroups for 256 CUs and measured fastest.
-//   * The four partial tiles are summed through LDS in a fixed order (deterministic), the
-//     scale/shift/ReLU epilogue is applied and each output row is written once, coalesced.
+// One workgroup (4 wave64) owns a tile of TM output rows and all Cout columns.
+//   * The tile's neighbour lists nbr[k][row0 .. row0+TM) are staged in LDS and compacted per offset
+//     with wave64 ballot + popcount: pair list k = the (input row, local output row) pairs of the rows
+//     that really have a neighbour at offset k.  Only those rows enter an MFMA block, so the matrix
+//     cores do not multiply the zero rows a dense [TM x K*Cin] gather matrix would be half full of.
+//   * Non-empty offsets are dealt round-robin to the four waves (split-K over offsets): tiles x 4 waves
+//     is what fills 256 CUs with a ~17k-row problem.
+//   * A wave gathers 16 pairs per MFMA block straight into A-operand registers: lane (i = lane%16,
+//     q = lane/16) loads 16 bytes = channels 16g+4q .. 16g+4q+3 of pair i's input row, i.e. every row is
+//     read as 64-byte segments.  The weights were reordered on the host so that the B operand of the same
+//     four MFMA steps is one 16-byte load per lane; one pass over W[k] serves all blocks of the offset.
+//     Next offset's rows and next chunk's weights are in flight while the current MFMAs issue.
+//   * v_mfma_f32_16x16x4_f32 accumulates a block in FP32 registers (weights as the A operand, gathered
+//     rows as B, so a lane ends up with four consecutive output channels of one pair); the block is then
+//     added into the wave's private partial tile in LDS at the pairs' output rows with 16-byte
+//     read-modify-writes (only this wave touches its partial and LDS keeps a wave's operations in order,
+//     so the sum order is fixed; LDS float atomics measured several times slower).
+//   * The four partial tiles are summed in a fixed order, scale/shift/ReLU is applied and each output
+//     row is written once, coalesced.  No global atomics; results are bit-identical run to run.
 #include "kernels.h"
 
 namespace sessd {
@@ -27,12 +32,13 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 #ifndef SESSD_MFMA_WAVES
 #define SESSD_MFMA_WAVES 4
 #endif
-#ifndef SESSD_MFMA_RB
-#define SESSD_MFMA_RB 1
+#ifndef SESSD_MFMA_TM
+#define SESSD_MFMA_TM 32
 #endif
 constexpr int kWaves = SESSD_MFMA_WAVES;
-constexpr int kRB = SESSD_MFMA_RB;   // 16-row MFMA blocks per wave
-constexpr int kTileRows = kRB * 16;
+constexpr int kTileRows = SESSD_MFMA_TM;   // output rows per workgroup (32 or 64)
+constexpr int kMaxBlk = kTileRows / 16;    // MFMA row blocks an offset can need
+constexpr int kMaxK = 27;
 
 template <int CIN, int COUT>
 __global__ void __launch_bounds__(kWaves * 64)
@@ -42,7 +48,9 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
     constexpr int G = CIN / 16;    // 16-channel chunks of the inner dimension
     constexpr int NB = COUT / 16;  // 16-column blocks
     constexpr int LDP = COUT + 4;  // padded row stride of the partial tiles in LDS
-    __shared__ int32_t s_nbr[27 * kTileRows];
+    __shared__ int32_t s_in[kMaxK * kTileRows];   // compacted pair lists: input row ...
+    __shared__ uint8_t s_row[kMaxK * kTileRows];  // ... and local output row of pair j of offset k
+    __shared__ int32_t s_cnt[kMaxK + 5];          // pairs per offset
     __shared__ float s_part[kWaves * kTileRows * LDP];
 
     const int row0 = blockIdx.x * kTileRows;
@@ -53,113 +61,151 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    for (int t = tid; t < K * kTileRows; t += kWaves * 64) {
-        const int k = t / kTileRows, r = t % kTileRows;
+
+    // ---- stage + compact: each half wave (TM = 32) or wave (TM = 64) owns one offset per step ----
+    constexpr int kPerWave = 64 / kTileRows;  // offsets a wave compacts per step
+    for (int k0 = wave * kPerWave; k0 < K; k0 += kWaves * kPerWave) {
+        const int k = k0 + lane / kTileRows;
+        const int r = lane % kTileRows;
         const int row = row0 + r;
-        s_nbr[t] = row < n ? nbr[(size_t)k * max_voxels + row] : -1;
+        const int v = (k < K && row < n) ? nbr[(size_t)k * max_voxels + row] : -1;
+        const uint64_t m = __ballot(v >= 0);
+        const uint64_t seg = kTileRows == 64 ? m : (m >> (lane & 32)) & 0xffffffffull;  // my offset's rows
+        if (v >= 0) {
+            const int j = __popcll(seg & ((1ull << r) - 1ull));
+            s_in[k * kTileRows + j] = v;
+            s_row[k * kTileRows + j] = (uint8_t)r;
+        }
+        if (r == 0 && k < K) s_cnt[k] = __popcll(seg);
     }
+    // zero this wave's partial tile
+    float* part = s_part + wave * kTileRows * LDP;
+    for (int t = lane; t < kTileRows * LDP / 4; t += 64) reinterpret_cast<float4*>(part)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
 
-    v4f acc[kRB][NB];
-#pragma unroll
-    for (int rb = 0; rb < kRB; ++rb)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) acc[rb][nb] = (v4f){0.f, 0.f, 0.f, 0.f};
-
-    const int i = lane & 15;  // row inside a 16-row block
+    const int i = lane & 15;  // pair inside a 16-pair block
     const int q = lane >> 4;  // 4-channel group inside a 16-channel chunk
 
-    // offsets this wave handles: the non-empty ones of the tile, dealt round-robin to the four waves;
-    // bit k of rb_mask[rb] = "16-row block rb has a neighbour at offset k" (all wave-uniform)
-    uint32_t my_mask = 0, rb_mask[kRB];
-#pragma unroll
-    for (int rb = 0; rb < kRB; ++rb) rb_mask[rb] = 0;
+    // offsets this wave handles: the non-empty ones, dealt round-robin (all wave-uniform)
+    uint32_t my_mask = 0;
     {
         int live = 0;
-        for (int k = 0; k < K; ++k) {
-            bool any = false;
-#pragma unroll
-            for (int rb = 0; rb < kRB; ++rb) {
-                const bool any_rb = __ballot(s_nbr[k * kTileRows + rb * 16 + i] >= 0) != 0ull;
-                if (any_rb) rb_mask[rb] |= 1u << k;
-                any = any || any_rb;
-            }
-            if (any) {
+        for (int k = 0; k < K; ++k)
+            if (s_cnt[k] > 0) {
                 if ((live % kWaves) == wave) my_mask |= 1u << k;
                 ++live;
             }
-        }
     }
 
-    // Software pipeline: the gathered rows of the NEXT offset and the weights of the NEXT 16-channel
-    // chunk are in flight while the MFMAs of the current chunk issue.
     const float4* wp4 = reinterpret_cast<const float4*>(Wp) + lane;
-    auto load_a = [&](int k, float4 (&a)[kRB][G]) {
+    // gathered rows of all blocks of offset k -> A-operand registers (zeros for the padding pairs)
+    auto load_a = [&](int k, int cnt, float4 (&a)[kMaxBlk][G]) {
 #pragma unroll
-        for (int rb = 0; rb < kRB; ++rb) {
-            const int idx = s_nbr[k * kTileRows + rb * 16 + i];
-            const float4* src = reinterpret_cast<const float4*>(in + (size_t)(idx < 0 ? 0 : idx) * CIN + q * 4);
+        for (int blk = 0; blk < kMaxBlk; ++blk) {
+            const int j = blk * 16 + i;
+            const bool live = j < cnt;
+            const int idx = live ? s_in[k * kTileRows + j] : 0;
+            const float4* src = reinterpret_cast<const float4*>(in + (size_t)idx * CIN + q * 4);
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (idx >= 0) v = src[g * 4];
-                a[rb][g] = v;
+#ifdef SESSD_EXP_NO_LOADS
+                v.x = (float)idx;
+#else
+                if (live) v = src[g * 4];
+#endif
+                a[blk][g] = v;
             }
         }
     };
     auto load_b = [&](int k, int g, float4 (&b)[NB]) {
         const float4* wk = wp4 + ((size_t)k * G + g) * NB * 64;
 #pragma unroll
+#ifdef SESSD_EXP_NO_LOADS
+        for (int nb = 0; nb < NB; ++nb) b[nb] = make_float4((float)(k + g), 1.f, 2.f, (float)nb);
+#else
         for (int nb = 0; nb < NB; ++nb) b[nb] = wk[nb * 64];
+#endif
     };
 
     int k_cur = my_mask ? __ffs(my_mask) - 1 : -1;
     my_mask &= my_mask - 1;
-    float4 a_cur[kRB][G], a_nxt[kRB][G], b_cur[NB], b_nxt[NB];
+    float4 a_cur[kMaxBlk][G], a_nxt[kMaxBlk][G], b_cur[NB], b_nxt[NB];
+    int cnt_cur = 0, cnt_nxt = 0;
     if (k_cur >= 0) {
-        load_a(k_cur, a_cur);
+        cnt_cur = s_cnt[k_cur];
+        load_a(k_cur, cnt_cur, a_cur);
         load_b(k_cur, 0, b_cur);
     }
     while (k_cur >= 0) {
         const int k_nxt = my_mask ? __ffs(my_mask) - 1 : -1;
         my_mask &= my_mask - 1;
-        if (k_nxt >= 0) load_a(k_nxt, a_nxt);
+        if (k_nxt >= 0) {
+            cnt_nxt = s_cnt[k_nxt];
+            load_a(k_nxt, cnt_nxt, a_nxt);
+        }
+        v4f acc[kMaxBlk][NB];
+#pragma unroll
+        for (int blk = 0; blk < kMaxBlk; ++blk)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) acc[blk][nb] = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             if (g + 1 < G) load_b(k_cur, g + 1, b_nxt);
             else if (k_nxt >= 0) load_b(k_nxt, 0, b_nxt);
 #pragma unroll
-            for (int rb = 0; rb < kRB; ++rb) {
-                if (!((rb_mask[rb] >> k_cur) & 1u)) continue;  // wave-uniform: block has no neighbour here
-                const float av[4] = {a_cur[rb][g].x, a_cur[rb][g].y, a_cur[rb][g].z, a_cur[rb][g].w};
+            for (int blk = 0; blk < kMaxBlk; ++blk) {
+                if (blk * 16 >= cnt_cur) continue;  // wave-uniform: this offset has fewer pairs
+                const float av[4] = {a_cur[blk][g].x, a_cur[blk][g].y, a_cur[blk][g].z, a_cur[blk][g].w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb) {
                         const float bv[4] = {b_cur[nb].x, b_cur[nb].y, b_cur[nb].z, b_cur[nb].w};
-                        acc[rb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[e], bv[e], acc[rb][nb], 0, 0, 0);
+#ifdef SESSD_EXP_NO_MFMA
+                        acc[blk][nb][0] += av[e] + bv[e];
+#else
+                        acc[blk][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(bv[e], av[e], acc[blk][nb], 0, 0, 0);
+#endif
                     }
             }
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) b_cur[nb] = b_nxt[nb];
         }
+        // block results -> partial tile.  The weights are the MFMA's A operand and the gathered rows its
+        // B operand, so D is the transposed block: lane (pair j = lane%16, q = lane/16) holds output
+        // channels 16nb+4q .. +3 of pair j -- one 16-byte LDS read-modify-write per column block.
 #pragma unroll
-        for (int rb = 0; rb < kRB; ++rb)
+        for (int blk = 0; blk < kMaxBlk; ++blk) {
+            if (blk * 16 >= cnt_cur) continue;
+            const int j = blk * 16 + i;
+            if (j < cnt_cur) {
+                float* dst = part + (int)s_row[k_cur * kTileRows + j] * LDP + q * 4;
+#ifndef SESSD_EXP_NO_ACCUM
 #pragma unroll
-            for (int g = 0; g < G; ++g) a_cur[rb][g] = a_nxt[rb][g];
+                for (int nb = 0; nb < NB; ++nb) {
+                    float4 v = *reinterpret_cast<float4*>(dst + nb * 16);
+                    v.x += acc[blk][nb][0];
+                    v.y += acc[blk][nb][1];
+                    v.z += acc[blk][nb][2];
+                    v.w += acc[blk][nb][3];
+                    *reinterpret_cast<float4*>(dst + nb * 16) = v;
+                }
+#else
+                float t = 0.f;
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) t += acc[blk][nb][0] + acc[blk][nb][1] + acc[blk][nb][2] + acc[blk][nb][3];
+                if (t == 123.f) dst[0] = 1.f;
+#endif
+            }
+        }
+#pragma unroll
+        for (int blk = 0; blk < kMaxBlk; ++blk)
+#pragma unroll
+            for (int g = 0; g < G; ++g) a_cur[blk][g] = a_nxt[blk][g];
         k_cur = k_nxt;
+        cnt_cur = cnt_nxt;
     }
-
-    // partial tile of this wave -> LDS.  D layout of the 16x16 MFMA: lane holds column lane%16 of rows
-    // 4*(lane/16) .. +3.
-    float* part = s_part + wave * kTileRows * LDP;
-#pragma unroll
-    for (int rb = 0; rb < kRB; ++rb)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                part[(rb * 16 + q * 4 + r) * LDP + nb * 16 + i] = acc[rb][nb][r];
     __syncthreads();
 
     // fixed-order sum of the four partials, epilogue, coalesced 16-byte stores
