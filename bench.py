@@ -79,6 +79,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch kernels directly instead of replaying a hipGraph")
     ap.add_argument("--no-share", action="store_true", help="every SubM layer rebuilds its rulebook (as the reference does)")
     ap.add_argument("--pad-rows", action="store_true", help="write rows >= voxel_num of every tensor (reference behaviour)")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="single stream: do not run the rulebook builds concurrently with the GEMMs of earlier layers")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--profile-steps", type=int, default=50)
     ap.add_argument("--calibrate-mb", type=int, default=0,
@@ -102,7 +104,7 @@ def main():
     max_points = args.points
     pipe = api.Pipeline(layers, W, max_points, args.max_voxels, feature_dtype=args.dtype,
                         share_rulebooks=not args.no_share, skip_pad_rows=not args.pad_rows,
-                        use_graph=not args.no_graph)
+                        use_graph=not args.no_graph, overlap_streams=not args.no_overlap)
     points = torch.as_tensor(pts).to(dev)
     size = torch.tensor([len(pts)], dtype=torch.int32, device=dev)
     dense = pipe.new_dense(dev)
@@ -188,7 +190,7 @@ def main():
         "config": {"workload": "config 3: %d-point seeded synthetic LiDAR frame (seed %d), %d voxels, reference 14-layer "
                                "SpMiddleFHD backbone (10 SubM + 4 SparseConv, BN folded + ReLU), sparse2Dense to 128x200x176"
                                % (len(pts), args.seed, n_vox),
-                   "max_voxels": args.max_voxels, "graph": not args.no_graph, "share_rulebooks": not args.no_share,
+                   "max_voxels": args.max_voxels, "graph": not args.no_graph, "overlap_streams": not args.no_overlap, "share_rulebooks": not args.no_share,
                    "pad_rows": args.pad_rows, "n_layers": len(layers)},
         "roofline": roof,
         "frame": {"frames_per_s": round(1e3 / ms_per_frame, 1), "algorithmic_gflop": round(tot_flops / 1e9, 3),

@@ -64,6 +64,60 @@ conv_valu_generic(const Tin* __restrict__ in, Tout* __restrict__ out, const Tw* 
     out[e] = from_f32<Tout>(apply_epilogue(acc, c, scale, shift, relu));
 }
 
+// First layer of the backbone (voxel means, Cin = 4): the inner dimension is too thin for MFMA tiles
+// (4 per offset).  One thread owns four output channels of one row; the whole weight tensor
+// (K*4*Cout floats, < 14 KB) sits in LDS, a gathered input row is one 16-byte load shared by the
+// row's threads.
+template <typename Tout, int COUT>
+__global__ void __launch_bounds__(kBlock)
+conv_valu_cin4(const float* __restrict__ in, Tout* __restrict__ out, const float* __restrict__ W,
+               const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
+               const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad) {
+    constexpr int TPR = COUT / 4;         // threads per row
+    constexpr int ROWS = kBlock / TPR;    // rows per block
+    __shared__ float4 s_w[27 * 4 * TPR];  // [k][j][c4]
+    for (int t = threadIdx.x; t < K * 4 * TPR; t += kBlock) s_w[t] = reinterpret_cast<const float4*>(W)[t];
+    __syncthreads();
+    const int row = blockIdx.x * ROWS + threadIdx.x / TPR;
+    const int c4 = threadIdx.x % TPR;
+    if (row >= max_voxels) return;
+    int n = *num_out;
+    n = n < 0 ? 0 : (n > max_voxels ? max_voxels : n);
+    if (row >= n && !write_pad) return;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (row < n) {
+        for (int k = 0; k < K; ++k) {
+            const int idx = nbr[(size_t)k * max_voxels + row];
+            if (idx < 0) continue;
+            const float4 x = reinterpret_cast<const float4*>(in)[idx];
+            const float4* w = s_w + k * 4 * TPR + c4;
+            float4 s;
+            s.x = x.x * w[0].x; s.y = x.x * w[0].y; s.z = x.x * w[0].z; s.w = x.x * w[0].w;
+            s.x = fmaf(x.y, w[TPR].x, s.x); s.y = fmaf(x.y, w[TPR].y, s.y); s.z = fmaf(x.y, w[TPR].z, s.z); s.w = fmaf(x.y, w[TPR].w, s.w);
+            s.x = fmaf(x.z, w[2 * TPR].x, s.x); s.y = fmaf(x.z, w[2 * TPR].y, s.y); s.z = fmaf(x.z, w[2 * TPR].z, s.z); s.w = fmaf(x.z, w[2 * TPR].w, s.w);
+            s.x = fmaf(x.w, w[3 * TPR].x, s.x); s.y = fmaf(x.w, w[3 * TPR].y, s.y); s.z = fmaf(x.w, w[3 * TPR].z, s.z); s.w = fmaf(x.w, w[3 * TPR].w, s.w);
+            acc.x += s.x; acc.y += s.y; acc.z += s.z; acc.w += s.w;
+        }
+    }
+    const int c = c4 * 4;
+    float o[4] = {acc.x, acc.y, acc.z, acc.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = apply_epilogue(o[e], c + e, scale, shift, relu);
+    Tout* dst = out + (size_t)row * COUT + c;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) dst[e] = from_f32<Tout>(o[e]);
+}
+
+template <typename Tout, int COUT>
+int launch_cin4(const GemmArgs& a, hipStream_t stream) {
+    constexpr int ROWS = kBlock / (COUT / 4);
+    hipLaunchKernelGGL((conv_valu_cin4<Tout, COUT>), dim3(ceil_div(a.max_voxels, ROWS)), dim3(kBlock), 0, stream,
+                       static_cast<const float*>(a.in_feat), static_cast<Tout*>(a.out_feat), a.w_f32, a.nbr,
+                       a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows);
+    SESSD_HIP_TRY(hipGetLastError());
+    return SESSD_OK;
+}
+
 template <typename Tin, typename Tw, typename Tout>
 int launch_generic(const GemmArgs& a, const Tw* w, hipStream_t stream) {
     const int64_t elems = (int64_t)a.max_voxels * a.cout;
@@ -143,6 +197,12 @@ int launch_gather_gemm(const GemmArgs& a, hipStream_t stream) {
     if (!a.force_valu) {
         const int rc = launch_mfma(a, stream);
         if (rc != SESSD_E_UNSUPPORTED) return rc;  // launched (or failed for good)
+    }
+    if (!a.force_valu && a.cin == 4 && a.K <= 27 && a.in_type == SESSD_FLOAT &&
+        !(reinterpret_cast<uintptr_t>(a.in_feat) & 15)) {
+        // (when the output is FP16 the weights are still FP32 here: the voxel means are FP32 inputs)
+        if (a.cout == 16 && a.out_type == SESSD_FLOAT) return launch_cin4<float, 16>(a, stream);
+        if (a.cout == 32 && a.out_type == SESSD_FLOAT) return launch_cin4<float, 32>(a, stream);
     }
     if (a.in_type == SESSD_FLOAT && a.out_type == SESSD_FLOAT)
         return launch_generic<float, float, float>(a, a.w_f32, stream);

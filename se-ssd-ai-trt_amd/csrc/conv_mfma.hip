@@ -2,7 +2,9 @@
 //
 //     out[o][:] = epilogue( sum_k  in[nbr[k][o]][:] @ W[k] )
 //
-// One workgroup (4 wave64) owns a tile of TM output rows and all Cout columns.
+// One workgroup (4 wave64) owns a tile of output rows and all Cout columns.  The tile height is chosen
+// per launch from the device-side row count so that every CU gets the same number of tiles
+// (tile_height()).
 //   * The tile's neighbour lists nbr[k][row0 .. row0+TM) are staged in LDS and compacted per offset
 //     with wave64 ballot + popcount: pair list k = the (input row, local output row) pairs of the rows
 //     that really have a neighbour at offset k.  Only those rows enter an MFMA block, so the matrix
@@ -35,16 +37,33 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 #ifndef SESSD_MFMA_TM
 #define SESSD_MFMA_TM 32
 #endif
+#ifndef SESSD_MFMA_TARGET
+#define SESSD_MFMA_TARGET 32
+#endif
 constexpr int kWaves = SESSD_MFMA_WAVES;
-constexpr int kTileRows = SESSD_MFMA_TM;   // output rows per workgroup (32 or 64)
-constexpr int kMaxBlk = kTileRows / 16;    // MFMA row blocks an offset can need
+constexpr int kTileRows = SESSD_MFMA_TM;      // capacity: most output rows a workgroup can own (<= 64)
+constexpr int kTargetRows = SESSD_MFMA_TARGET;  // tile height aimed for when choosing tiles per CU
+constexpr int kMaxBlk = (kTileRows + 15) / 16;  // MFMA row blocks an offset can need
 constexpr int kMaxK = 27;
+
+// Tile height for `n` active rows on `num_cu` compute units: the rows are split into num_cu * r tiles
+// of equal height, r = the smallest tiles-per-CU count that keeps the height at or below the target.
+// Every CU then gets the same number of tiles (a fixed 32-row tiling leaves e.g. 529 tiles for 256 CUs:
+// some CUs run three tiles, most two, and the kernel lasts as long as the three).
+static_assert(kTargetRows <= kTileRows && kTileRows <= 64, "tile height must fit the capacity and one wave");
+__host__ __device__ inline int tile_height(int n, int num_cu) {
+    if (n <= 0) return kTileRows;
+    const int r = (n + num_cu * kTargetRows - 1) / (num_cu * kTargetRows);
+    int h = (n + num_cu * r - 1) / (num_cu * r);
+    return h > kTileRows ? kTileRows : (h < 1 ? 1 : h);
+}
 
 template <int CIN, int COUT>
 __global__ void __launch_bounds__(kWaves * 64)
 conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float* __restrict__ Wp,
               const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
-              const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad) {
+              const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad,
+              int num_cu) {
     constexpr int G = CIN / 16;    // 16-channel chunks of the inner dimension
     constexpr int NB = COUT / 16;  // 16-column blocks
     constexpr int LDP = COUT + 4;  // padded row stride of the partial tiles in LDS
@@ -53,34 +72,51 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
     __shared__ int32_t s_cnt[kMaxK + 5];          // pairs per offset
     __shared__ float s_part[kWaves * kTileRows * LDP];
 
-    const int row0 = blockIdx.x * kTileRows;
     int n = *num_out;
     n = n < 0 ? 0 : (n > max_voxels ? max_voxels : n);
-    if (row0 >= n && !write_pad) return;
-
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    constexpr int kVecPerRow = COUT / 4;
 
-    // ---- stage + compact: each half wave (TM = 32) or wave (TM = 64) owns one offset per step ----
-    constexpr int kPerWave = 64 / kTileRows;  // offsets a wave compacts per step
-    for (int k0 = wave * kPerWave; k0 < K; k0 += kWaves * kPerWave) {
-        const int k = k0 + lane / kTileRows;
-        const int r = lane % kTileRows;
-        const int row = row0 + r;
-        const int v = (k < K && row < n) ? nbr[(size_t)k * max_voxels + row] : -1;
+    // rows >= n: the reference zero-fills them (then BN+ReLU): epilogue(0), spread over all workgroups
+    if (write_pad) {
+        const int chunks = (max_voxels - n + kTileRows - 1) / kTileRows;
+        for (int c = blockIdx.x; c < chunks; c += gridDim.x)
+            for (int v = tid; v < kTileRows * kVecPerRow; v += kWaves * 64) {
+                const int row = n + c * kTileRows + v / kVecPerRow, c4 = (v % kVecPerRow) * 4;
+                if (row >= max_voxels) continue;
+                float o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float s = 0.f;
+                    if (scale) s = s * scale[c4 + e];
+                    if (shift) s = s + shift[c4 + e];
+                    if (relu) s = s > 0.f ? s : 0.f;
+                    o[e] = s;
+                }
+                *reinterpret_cast<float4*>(out + (size_t)row * COUT + c4) = make_float4(o[0], o[1], o[2], o[3]);
+            }
+    }
+    const int R = tile_height(n, num_cu);  // rows of this launch's tiles
+    const int row0 = blockIdx.x * R;
+    if (row0 >= n) return;
+    const int rows = n - row0 < R ? n - row0 : R;
+
+    // ---- stage + compact: a wave turns one offset's neighbour list into a pair list per step ----
+    for (int k = wave; k < K; k += kWaves) {
+        const int v = lane < rows ? nbr[(size_t)k * max_voxels + row0 + lane] : -1;
         const uint64_t m = __ballot(v >= 0);
-        const uint64_t seg = kTileRows == 64 ? m : (m >> (lane & 32)) & 0xffffffffull;  // my offset's rows
         if (v >= 0) {
-            const int j = __popcll(seg & ((1ull << r) - 1ull));
+            const int j = __popcll(m & ((1ull << lane) - 1ull));
             s_in[k * kTileRows + j] = v;
-            s_row[k * kTileRows + j] = (uint8_t)r;
+            s_row[k * kTileRows + j] = (uint8_t)lane;
         }
-        if (r == 0 && k < K) s_cnt[k] = __popcll(seg);
+        if (lane == 0) s_cnt[k] = __popcll(m);
     }
     // zero this wave's partial tile
     float* part = s_part + wave * kTileRows * LDP;
-    for (int t = lane; t < kTileRows * LDP / 4; t += 64) reinterpret_cast<float4*>(part)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int t = lane; t < rows * LDP / 4; t += 64) reinterpret_cast<float4*>(part)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
 
     const int i = lane & 15;  // pair inside a 16-pair block
@@ -130,12 +166,17 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
 
     int k_cur = my_mask ? __ffs(my_mask) - 1 : -1;
     my_mask &= my_mask - 1;
-    float4 a_cur[kMaxBlk][G], a_nxt[kMaxBlk][G], b_cur[NB], b_nxt[NB];
+    // Pipeline: the gathered rows of the NEXT offset are loaded at the top of the current one; the
+    // weight registers of chunk g are refilled with the next offset's chunk g as soon as the MFMAs that
+    // read them have issued, so every weight load has a whole offset of MFMA work to hide behind
+    // without a second register set.
+    float4 a_cur[kMaxBlk][G], a_nxt[kMaxBlk][G], b[G][NB];
     int cnt_cur = 0, cnt_nxt = 0;
     if (k_cur >= 0) {
         cnt_cur = s_cnt[k_cur];
         load_a(k_cur, cnt_cur, a_cur);
-        load_b(k_cur, 0, b_cur);
+#pragma unroll
+        for (int g = 0; g < G; ++g) load_b(k_cur, g, b[g]);
     }
     while (k_cur >= 0) {
         const int k_nxt = my_mask ? __ffs(my_mask) - 1 : -1;
@@ -151,8 +192,6 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
             for (int nb = 0; nb < NB; ++nb) acc[blk][nb] = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            if (g + 1 < G) load_b(k_cur, g + 1, b_nxt);
-            else if (k_nxt >= 0) load_b(k_nxt, 0, b_nxt);
 #pragma unroll
             for (int blk = 0; blk < kMaxBlk; ++blk) {
                 if (blk * 16 >= cnt_cur) continue;  // wave-uniform: this offset has fewer pairs
@@ -161,16 +200,11 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
                 for (int e = 0; e < 4; ++e)
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb) {
-                        const float bv[4] = {b_cur[nb].x, b_cur[nb].y, b_cur[nb].z, b_cur[nb].w};
-#ifdef SESSD_EXP_NO_MFMA
-                        acc[blk][nb][0] += av[e] + bv[e];
-#else
+                        const float bv[4] = {b[g][nb].x, b[g][nb].y, b[g][nb].z, b[g][nb].w};
                         acc[blk][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(bv[e], av[e], acc[blk][nb], 0, 0, 0);
-#endif
                     }
             }
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) b_cur[nb] = b_nxt[nb];
+            if (k_nxt >= 0) load_b(k_nxt, g, b[g]);
         }
         // block results -> partial tile.  The weights are the MFMA's A operand and the gathered rows its
         // B operand, so D is the transposed block: lane (pair j = lane%16, q = lane/16) holds output
@@ -209,11 +243,8 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
     __syncthreads();
 
     // fixed-order sum of the four partials, epilogue, coalesced 16-byte stores
-    constexpr int kVecPerRow = COUT / 4;
-    for (int v = tid; v < kTileRows * kVecPerRow; v += kWaves * 64) {
+    for (int v = tid; v < rows * kVecPerRow; v += kWaves * 64) {
         const int r = v / kVecPerRow, c4 = (v % kVecPerRow) * 4;
-        const int row = row0 + r;
-        if (row >= max_voxels || (row >= n && !write_pad)) continue;
         float o[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -225,17 +256,33 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
             if (relu) s = s > 0.f ? s : 0.f;
             o[e] = s;
         }
-        *reinterpret_cast<float4*>(out + (size_t)row * COUT + c4) = make_float4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<float4*>(out + (size_t)(row0 + r) * COUT + c4) = make_float4(o[0], o[1], o[2], o[3]);
     }
+}
+
+int compute_units() {
+    static int cu = 0;
+    if (cu == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+            cu = v;
+        else
+            cu = 256;
+    }
+    return cu;
 }
 
 template <int CIN, int COUT>
 int launch_f32(const GemmArgs& a, hipStream_t stream) {
-    const unsigned blocks = (unsigned)ceil_div(a.max_voxels, kTileRows);
+    const int num_cu = compute_units();
+    // tile_height() never cuts n <= max_voxels rows into more than num_cu * r_max tiles
+    const int r_max = ceil_div(a.max_voxels, (int64_t)num_cu * kTargetRows);
+    const unsigned blocks = (unsigned)(num_cu * (r_max < 1 ? 1 : r_max));
     hipLaunchKernelGGL((conv_mfma_f32<CIN, COUT>), dim3(blocks), dim3(kWaves * 64), 0, stream,
                        static_cast<const float*>(a.in_feat), static_cast<float*>(a.out_feat),
                        static_cast<const float*>(a.w_packed), a.nbr, a.num_out, a.max_voxels, a.K, a.scale,
-                       a.shift, a.relu, a.write_pad_rows);
+                       a.shift, a.relu, a.write_pad_rows, num_cu);
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;
 }

@@ -67,6 +67,12 @@ struct Pipeline {
     void* g_dense = nullptr;
     int graph_nodes = -1;
 
+    // two-stream schedule: coordinate chain (voxelizer + rulebook builds) on `aux`, feature chain on the
+    // caller's stream; ev_build[l] = "rulebook of layer l is ready"
+    hipStream_t aux = nullptr;
+    hipEvent_t ev_start = nullptr, ev_vg = nullptr;
+    std::vector<hipEvent_t> ev_build;
+
     // profiling: one event per segment boundary (see sessd_pipeline_enqueue_timed)
     std::vector<hipEvent_t> events;
     DeviceBuffer stats;  // u32[32] scratch for per-offset pair counts
@@ -75,6 +81,65 @@ struct Pipeline {
         if (graph_exec) (void)hipGraphExecDestroy(graph_exec);
         if (graph) (void)hipGraphDestroy(graph);
         for (hipEvent_t e : events) (void)hipEventDestroy(e);
+        for (hipEvent_t e : ev_build)
+            if (e) (void)hipEventDestroy(e);
+        if (ev_start) (void)hipEventDestroy(ev_start);
+        if (ev_vg) (void)hipEventDestroy(ev_vg);
+        if (aux) (void)hipStreamDestroy(aux);
+    }
+
+    // The rulebooks depend only on coordinates, the GEMMs on rulebooks + features.  The coordinate chain
+    // (voxelizer, then every layer's rulebook build in order) runs on `aux`; the GEMM chain on `stream`
+    // waits per layer for the rulebook it needs, so the small build kernels of later layers overlap the
+    // GEMMs of earlier ones.  Under stream capture the fork/join becomes two branches of the graph.
+    int enqueueOverlapped(const void* points, const void* points_size, void* dense, hipStream_t stream) {
+        SESSD_HIP_TRY(hipEventRecord(ev_start, stream));
+        SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_start, 0));
+        const void* vin[2] = {points, points_size};
+        void* vout[3] = {vg_voxels.p, vg_coors.p, vg_num.p};
+        SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, aux));
+        SESSD_HIP_TRY(hipEventRecord(ev_vg, aux));
+        const int32_t* coors = static_cast<const int32_t*>(vg_coors.p);
+        const int32_t* num = static_cast<const int32_t*>(vg_num.p);
+        for (size_t l = 0; l < stages.size(); ++l) {
+            ConvStage& st = *stages[l];
+            if (st.subm) {
+                if (st.rulebook_from >= 0) continue;
+                SESSD_TRY(st.subm->enqueueBuild(coors, num, st.ws.p, aux));
+            } else {
+                SESSD_TRY(st.sparse->enqueueBuild(coors, num, static_cast<int32_t*>(st.coors.p),
+                                                  static_cast<int32_t*>(st.num.p), st.ws.p, aux));
+                coors = static_cast<const int32_t*>(st.coors.p);
+                num = static_cast<const int32_t*>(st.num.p);
+            }
+            SESSD_HIP_TRY(hipEventRecord(ev_build[l], aux));
+        }
+        SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_vg, 0));
+        const void* feat = vg_voxels.p;
+        coors = static_cast<const int32_t*>(vg_coors.p);
+        num = static_cast<const int32_t*>(vg_num.p);
+        int last_waited = -1;
+        for (size_t l = 0; l < stages.size(); ++l) {
+            ConvStage& st = *stages[l];
+            const int owner = st.rulebook_from >= 0 ? st.rulebook_from : (int)l;
+            if (owner > last_waited) {
+                SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_build[owner], 0));
+                last_waited = owner;
+            }
+            if (st.subm) {
+                SESSD_TRY(st.subm->enqueueGemm(feat, st.feat.p, num, stages[owner]->ws.p, stream));
+            } else {
+                SESSD_TRY(st.sparse->enqueueGemm(feat, st.feat.p, static_cast<const int32_t*>(st.num.p), st.ws.p, stream));
+                coors = static_cast<const int32_t*>(st.coors.p);
+                num = static_cast<const int32_t*>(st.num.p);
+            }
+            feat = st.feat.p;
+        }
+        // every event of `aux` has been waited on by now (the last build is the last aux operation)
+        if (stages.empty()) SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_vg, 0));
+        const void* din[3] = {feat, coors, num};
+        void* dout[1] = {dense};
+        return s2d->enqueue(s2d_in, s2d_out, din, dout, s2d_ws.p, stream);
     }
 
     int enqueueDirect(const void* points, const void* points_size, void* dense, hipStream_t stream) {
@@ -233,6 +298,13 @@ static int build_pipeline(const sessd_pipeline_desc& d, Pipeline* P) {
     SESSD_TRY(P->s2d_ws.alloc(s2d->getWorkspaceSize(P->s2d_in, 3, P->s2d_out, 1)));
     total += P->s2d_ws.bytes;
     P->device_bytes = total;
+    if (d.overlap_streams) {
+        SESSD_HIP_TRY(hipStreamCreateWithFlags(&P->aux, hipStreamNonBlocking));
+        SESSD_HIP_TRY(hipEventCreateWithFlags(&P->ev_start, hipEventDisableTiming));
+        SESSD_HIP_TRY(hipEventCreateWithFlags(&P->ev_vg, hipEventDisableTiming));
+        P->ev_build.assign(P->stages.size(), nullptr);
+        for (auto& e : P->ev_build) SESSD_HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    }
     // the layer array of the caller need not outlive create()
     P->desc.layers = nullptr;
     P->desc.weights = P->desc.scale = P->desc.shift = nullptr;
@@ -303,14 +375,17 @@ int sessd_pipeline_enqueue(sessd_pipeline* h, const void* points, const void* po
     if (!h || !points || !points_size || !dense) return fail(SESSD_E_INVALID, "pipeline_enqueue: null argument");
     auto* P = reinterpret_cast<Pipeline*>(h);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (!P->desc.use_graph || stream == nullptr) return P->enqueueDirect(points, points_size, dense, stream);
+    auto run = [&](hipStream_t st) {
+        return P->aux ? P->enqueueOverlapped(points, points_size, dense, st) : P->enqueueDirect(points, points_size, dense, st);
+    };
+    if (!P->desc.use_graph || stream == nullptr) return run(stream);
     if (!P->graph_exec || P->g_points != points || P->g_size != points_size || P->g_dense != dense) {
         if (P->graph_exec) (void)hipGraphExecDestroy(P->graph_exec);
         if (P->graph) (void)hipGraphDestroy(P->graph);
         P->graph_exec = nullptr;
         P->graph = nullptr;
         SESSD_HIP_TRY(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
-        const int rc = P->enqueueDirect(points, points_size, dense, stream);
+        const int rc = run(stream);
         hipGraph_t g = nullptr;
         const hipError_t e = hipStreamEndCapture(stream, &g);
         if (rc != SESSD_OK) {

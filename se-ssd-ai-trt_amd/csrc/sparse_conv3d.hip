@@ -340,18 +340,14 @@ size_t SparseConv3dLayerPlugin::getWorkspaceSize(const sessd_tensor_desc*, int, 
 
 size_t SparseConv3dLayerPlugin::statusOffset() const { return carve(nullptr).meta_offset; }
 
-int SparseConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
-                                     const void* const* inputs, void* const* outputs, void* workspace,
-                                     hipStream_t stream) {
-    SESSD_TRY(conv_check_io(inputDesc, outputDesc, inputs, outputs, in_type_, out_type_, max_voxels_,
-                            in_channel_, out_channel_, "sparseconv3d.enqueue"));
-    if (!workspace || !outputs[1] || !outputs[2]) return fail(SESSD_E_INVALID, "sparseconv3d.enqueue: null pointer");
-    if (reinterpret_cast<uintptr_t>(outputs[1]) & 15)
-        return fail(SESSD_E_INVALID, "sparseconv3d.enqueue: output coors must be 16-byte aligned");
-    const int32_t* coors = static_cast<const int32_t*>(inputs[1]);
-    const int32_t* voxel_num = static_cast<const int32_t*>(inputs[2]);
-    int32_t* out_coors = static_cast<int32_t*>(outputs[1]);
-    int32_t* out_num = static_cast<int32_t*>(outputs[2]);
+// The two halves of enqueue (see SubmConv3dLayerPlugin::enqueueBuild): output sites + rulebook from the
+// coordinates, then the GEMM over the features.
+int SparseConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* voxel_num, int32_t* out_coors,
+                                          int32_t* out_num, void* workspace, hipStream_t stream) {
+    if (!coors || !voxel_num || !out_coors || !out_num || !workspace)
+        return fail(SESSD_E_INVALID, "sparseconv3d.build: null pointer");
+    if (reinterpret_cast<uintptr_t>(out_coors) & 15)
+        return fail(SESSD_E_INVALID, "sparseconv3d.build: output coors must be 16-byte aligned");
     const Layout L = carve(workspace);
     const HashTable t = make_hash(L.keys, L.vals, L.cap);
     SpParams P;
@@ -376,7 +372,26 @@ int SparseConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const s
                        L.n_blocks, out_coors, out_num, L.meta);
     hipLaunchKernelGGL(sp_scatter, grid, block, 0, stream, voxel_num, P, t, L.cand, L.nbr);
     SESSD_HIP_TRY(hipGetLastError());
-    return runGemm(inputs[0], outputs[0], L.nbr, out_num, stream);
+    return SESSD_OK;
+}
+
+int SparseConv3dLayerPlugin::enqueueGemm(const void* in_feat, void* out_feat, const int32_t* out_num,
+                                         const void* workspace, hipStream_t stream) {
+    if (!in_feat || !out_feat || !out_num || !workspace) return fail(SESSD_E_INVALID, "sparseconv3d.gemm: null pointer");
+    const Layout L = carve(const_cast<void*>(workspace));
+    return runGemm(in_feat, out_feat, L.nbr, out_num, stream);
+}
+
+int SparseConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
+                                     const void* const* inputs, void* const* outputs, void* workspace,
+                                     hipStream_t stream) {
+    SESSD_TRY(conv_check_io(inputDesc, outputDesc, inputs, outputs, in_type_, out_type_, max_voxels_,
+                            in_channel_, out_channel_, "sparseconv3d.enqueue"));
+    if (!workspace || !outputs[1] || !outputs[2]) return fail(SESSD_E_INVALID, "sparseconv3d.enqueue: null pointer");
+    int32_t* out_num = static_cast<int32_t*>(outputs[2]);
+    SESSD_TRY(enqueueBuild(static_cast<const int32_t*>(inputs[1]), static_cast<const int32_t*>(inputs[2]),
+                           static_cast<int32_t*>(outputs[1]), out_num, workspace, stream));
+    return enqueueGemm(inputs[0], outputs[0], out_num, workspace, stream);
 }
 
 int SparseConv3dLayerPlugin::exportRulebook(const void* workspace, int32_t* indice_pairs, uint32_t* indice_num,

@@ -219,18 +219,14 @@ size_t SubmConv3dLayerPlugin::getWorkspaceSize(const sessd_tensor_desc*, int, co
 
 size_t SubmConv3dLayerPlugin::statusOffset() const { return carve(nullptr).meta_offset; }
 
-int SubmConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
-                                   const void* const* inputs, void* const* outputs, void* workspace,
-                                   hipStream_t stream) {
-    SESSD_TRY(conv_check_io(inputDesc, outputDesc, inputs, outputs, in_type_, out_type_, max_voxels_,
-                            in_channel_, out_channel_, "submconv3d.enqueue"));
-    if (!workspace) return fail(SESSD_E_INVALID, "submconv3d.enqueue: workspace is null");
-    const int32_t* coors = static_cast<const int32_t*>(inputs[1]);
-    const int32_t* voxel_num = static_cast<const int32_t*>(inputs[2]);
+// The two halves of enqueue.  The rulebook depends only on the coordinates, the GEMM only on the
+// rulebook and the features: a pipeline may run the halves of different layers on different streams.
+int SubmConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* voxel_num, void* workspace,
+                                        hipStream_t stream) {
+    if (!coors || !voxel_num || !workspace) return fail(SESSD_E_INVALID, "submconv3d.build: null pointer");
     const Layout L = carve(workspace);
     const HashTable t = make_hash(L.keys, L.vals, L.cap);
     const Grid3 g{out_shape_x_, out_shape_y_, out_shape_z_};
-
     FillArgs f;
     f.add(L.keys, (uint64_t)L.cap * 2, kEmpty);
     f.add(L.meta, 4, 0);
@@ -241,7 +237,26 @@ int SubmConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const ses
     hipLaunchKernelGGL(subm_neighbours, dim3(row_blocks, kernel_volume_), dim3(kBlock), 0, stream, coors,
                        voxel_num, max_voxels_, g, ksize_, padding_, t, L.nbr);
     SESSD_HIP_TRY(hipGetLastError());
-    return runGemm(inputs[0], outputs[0], L.nbr, voxel_num, stream);
+    return SESSD_OK;
+}
+
+int SubmConv3dLayerPlugin::enqueueGemm(const void* in_feat, void* out_feat, const int32_t* voxel_num,
+                                       const void* rulebook_workspace, hipStream_t stream) {
+    if (!in_feat || !out_feat || !voxel_num || !rulebook_workspace)
+        return fail(SESSD_E_INVALID, "submconv3d.gemm: null pointer");
+    const Layout L = carve(const_cast<void*>(rulebook_workspace));
+    return runGemm(in_feat, out_feat, L.nbr, voxel_num, stream);
+}
+
+int SubmConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
+                                   const void* const* inputs, void* const* outputs, void* workspace,
+                                   hipStream_t stream) {
+    SESSD_TRY(conv_check_io(inputDesc, outputDesc, inputs, outputs, in_type_, out_type_, max_voxels_,
+                            in_channel_, out_channel_, "submconv3d.enqueue"));
+    if (!workspace) return fail(SESSD_E_INVALID, "submconv3d.enqueue: workspace is null");
+    const int32_t* voxel_num = static_cast<const int32_t*>(inputs[2]);
+    SESSD_TRY(enqueueBuild(static_cast<const int32_t*>(inputs[1]), voxel_num, workspace, stream));
+    return enqueueGemm(inputs[0], outputs[0], voxel_num, workspace, stream);
 }
 
 int SubmConv3dLayerPlugin::enqueueShared(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
@@ -250,8 +265,7 @@ int SubmConv3dLayerPlugin::enqueueShared(const sessd_tensor_desc* inputDesc, con
     SESSD_TRY(conv_check_io(inputDesc, outputDesc, inputs, outputs, in_type_, out_type_, max_voxels_,
                             in_channel_, out_channel_, "submconv3d.enqueue_shared"));
     if (!rulebook_workspace) return fail(SESSD_E_INVALID, "submconv3d.enqueue_shared: rulebook workspace is null");
-    const Layout L = carve(const_cast<void*>(rulebook_workspace));
-    return runGemm(inputs[0], outputs[0], L.nbr, static_cast<const int32_t*>(inputs[2]), stream);
+    return enqueueGemm(inputs[0], outputs[0], static_cast<const int32_t*>(inputs[2]), rulebook_workspace, stream);
 }
 
 int SubmConv3dLayerPlugin::exportRulebook(const void* workspace, int32_t* indice_pairs, uint32_t* indice_num,

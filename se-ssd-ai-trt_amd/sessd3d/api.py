@@ -349,7 +349,7 @@ class Pipeline:
     def __init__(self, layers, weights: B.Weights, max_points, max_voxels=B.MAX_VOXELS, point_features=4,
                  feature_dtype="fp32", relu=True, share_rulebooks=True, skip_pad_rows=False, use_graph=False,
                  dense_size_xyz=B.DENSE_SIZE_XYZ, max_pts_per_voxel=B.MAX_NUM_POINTS_PER_VOXEL,
-                 use_epilogue=True):
+                 use_epilogue=True, overlap_streams=False):
         torch = _torch()
         self.layers = list(layers)
         self.max_points, self.max_voxels = max_points, max_voxels
@@ -376,6 +376,7 @@ class Pipeline:
         d.share_rulebooks = int(share_rulebooks)
         d.flags = D.SESSD_FLAG_SKIP_PAD_ROWS if skip_pad_rows else 0
         d.use_graph = int(use_graph)
+        d.overlap_streams = int(overlap_streams)
         self.dense_shape = (c_last * dense_size_xyz[2], dense_size_xyz[1], dense_size_xyz[0])
         self.h = C.c_void_p()
         check(lib().sessd_pipeline_create(C.byref(d), C.byref(self.h)))

@@ -74,7 +74,14 @@ def test_full_backbone_config3_frame_and_graph_replay():
     assert 15000 < ref["counts"][0] < 19000
     eager = to_np(dense).copy()
 
-    gpipe = api.Pipeline(layers, W, 20000, 60000, share_rulebooks=True, skip_pad_rows=True, use_graph=True)
+    # two-stream schedule, eager: same bits as the single-stream run
+    opipe, odense, _ = run_pipeline(pts, layers, W, 20000, 60000, share_rulebooks=True, skip_pad_rows=True,
+                                    overlap_streams=True)
+    assert np.array_equal(to_np(odense), eager), "two-stream schedule differs from the single-stream result"
+    assert opipe.status() == 0
+
+    gpipe = api.Pipeline(layers, W, 20000, 60000, share_rulebooks=True, skip_pad_rows=True, use_graph=True,
+                         overlap_streams=True)
     p, n = points_input(pts, 20000)
     gd = gpipe.new_dense()
     stream = torch.cuda.Stream()
