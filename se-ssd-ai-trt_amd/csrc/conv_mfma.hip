@@ -35,10 +35,10 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 #define SESSD_MFMA_WAVES 4
 #endif
 #ifndef SESSD_MFMA_TM
-#define SESSD_MFMA_TM 32
+#define SESSD_MFMA_TM 48
 #endif
 #ifndef SESSD_MFMA_TARGET
-#define SESSD_MFMA_TARGET 32
+#define SESSD_MFMA_TARGET 40
 #endif
 constexpr int kWaves = SESSD_MFMA_WAVES;
 constexpr int kTileRows = SESSD_MFMA_TM;      // capacity: most output rows a workgroup can own (<= 64)
