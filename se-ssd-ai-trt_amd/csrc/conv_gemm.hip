@@ -68,15 +68,16 @@ conv_valu_generic(const Tin* __restrict__ in, Tout* __restrict__ out, const Tw* 
 // (4 per offset).  One thread owns four output channels of one row; the whole weight tensor
 // (K*4*Cout floats, < 14 KB) sits in LDS, a gathered input row is one 16-byte load shared by the
 // row's threads.
-template <typename Tout, int COUT>
+template <typename Tw, typename Tout, int COUT>
 __global__ void __launch_bounds__(kBlock)
-conv_valu_cin4(const float* __restrict__ in, Tout* __restrict__ out, const float* __restrict__ W,
+conv_valu_cin4(const float* __restrict__ in, Tout* __restrict__ out, const Tw* __restrict__ W,
                const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
                const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad) {
     constexpr int TPR = COUT / 4;         // threads per row
     constexpr int ROWS = kBlock / TPR;    // rows per block
     __shared__ float4 s_w[27 * 4 * TPR];  // [k][j][c4]
-    for (int t = threadIdx.x; t < K * 4 * TPR; t += kBlock) s_w[t] = reinterpret_cast<const float4*>(W)[t];
+    for (int t = threadIdx.x; t < K * 4 * TPR; t += kBlock)
+        s_w[t] = make_float4(to_f32(W[4 * t]), to_f32(W[4 * t + 1]), to_f32(W[4 * t + 2]), to_f32(W[4 * t + 3]));
     __syncthreads();
     const int row = blockIdx.x * ROWS + threadIdx.x / TPR;
     const int c4 = threadIdx.x % TPR;
@@ -108,11 +109,11 @@ conv_valu_cin4(const float* __restrict__ in, Tout* __restrict__ out, const float
     for (int e = 0; e < 4; ++e) dst[e] = from_f32<Tout>(o[e]);
 }
 
-template <typename Tout, int COUT>
-int launch_cin4(const GemmArgs& a, hipStream_t stream) {
+template <typename Tw, typename Tout, int COUT>
+int launch_cin4(const GemmArgs& a, const Tw* w, hipStream_t stream) {
     constexpr int ROWS = kBlock / (COUT / 4);
-    hipLaunchKernelGGL((conv_valu_cin4<Tout, COUT>), dim3(ceil_div(a.max_voxels, ROWS)), dim3(kBlock), 0, stream,
-                       static_cast<const float*>(a.in_feat), static_cast<Tout*>(a.out_feat), a.w_f32, a.nbr,
+    hipLaunchKernelGGL((conv_valu_cin4<Tw, Tout, COUT>), dim3(ceil_div(a.max_voxels, ROWS)), dim3(kBlock), 0, stream,
+                       static_cast<const float*>(a.in_feat), static_cast<Tout*>(a.out_feat), w, a.nbr,
                        a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows);
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;
@@ -200,9 +201,11 @@ int launch_gather_gemm(const GemmArgs& a, hipStream_t stream) {
     }
     if (!a.force_valu && a.cin == 4 && a.K <= 27 && a.in_type == SESSD_FLOAT &&
         !(reinterpret_cast<uintptr_t>(a.in_feat) & 15)) {
-        // (when the output is FP16 the weights are still FP32 here: the voxel means are FP32 inputs)
-        if (a.cout == 16 && a.out_type == SESSD_FLOAT) return launch_cin4<float, 16>(a, stream);
-        if (a.cout == 32 && a.out_type == SESSD_FLOAT) return launch_cin4<float, 32>(a, stream);
+        // FP16 output = the FP16 configuration: half-rounded weights, as in every other layer
+        if (a.cout == 16 && a.out_type == SESSD_FLOAT) return launch_cin4<float, float, 16>(a, a.w_f32, stream);
+        if (a.cout == 32 && a.out_type == SESSD_FLOAT) return launch_cin4<float, float, 32>(a, a.w_f32, stream);
+        if (a.cout == 16 && a.out_type == SESSD_HALF) return launch_cin4<__half, __half, 16>(a, a.w_f16, stream);
+        if (a.cout == 32 && a.out_type == SESSD_HALF) return launch_cin4<__half, __half, 32>(a, a.w_f16, stream);
     }
     if (a.in_type == SESSD_FLOAT && a.out_type == SESSD_FLOAT)
         return launch_generic<float, float, float>(a, a.w_f32, stream);

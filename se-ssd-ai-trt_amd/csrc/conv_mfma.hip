@@ -1,28 +1,31 @@
-// conv_mfma.hip -- gather-GEMM on the matrix cores (gfx950 MFMA), FP32 features.
+// conv_mfma.hip -- gather-GEMM on the matrix cores (gfx950 MFMA), FP32 or FP16 features, FP32 accumulate.
 //
 //     out[o][:] = epilogue( sum_k  in[nbr[k][o]][:] @ W[k] )
 //
 // One workgroup (4 wave64) owns a tile of output rows and all Cout columns.  The tile height is chosen
 // per launch from the device-side row count so that every CU gets the same number of tiles
 // (tile_height()).
-//   * The tile's neighbour lists nbr[k][row0 .. row0+TM) are staged in LDS and compacted per offset
+//   * The tile's neighbour lists nbr[k][row0 .. row0+rows) are staged in LDS and compacted per offset
 //     with wave64 ballot + popcount: pair list k = the (input row, local output row) pairs of the rows
 //     that really have a neighbour at offset k.  Only those rows enter an MFMA block, so the matrix
-//     cores do not multiply the zero rows a dense [TM x K*Cin] gather matrix would be half full of.
+//     cores do not multiply the zero rows a dense [rows x K*Cin] gather matrix would be half full of.
 //   * Non-empty offsets are dealt round-robin to the four waves (split-K over offsets): tiles x 4 waves
 //     is what fills 256 CUs with a ~17k-row problem.
-//   * A wave gathers 16 pairs per MFMA block straight into A-operand registers: lane (i = lane%16,
-//     q = lane/16) loads 16 bytes = channels 16g+4q .. 16g+4q+3 of pair i's input row, i.e. every row is
-//     read as 64-byte segments.  The weights were reordered on the host so that the B operand of the same
-//     four MFMA steps is one 16-byte load per lane; one pass over W[k] serves all blocks of the offset.
-//     Next offset's rows and next chunk's weights are in flight while the current MFMAs issue.
-//   * v_mfma_f32_16x16x4_f32 accumulates a block in FP32 registers (weights as the A operand, gathered
-//     rows as B, so a lane ends up with four consecutive output channels of one pair); the block is then
-//     added into the wave's private partial tile in LDS at the pairs' output rows with 16-byte
-//     read-modify-writes (only this wave touches its partial and LDS keeps a wave's operations in order,
-//     so the sum order is fixed; LDS float atomics measured several times slower).
-//   * The four partial tiles are summed in a fixed order, scale/shift/ReLU is applied and each output
-//     row is written once, coalesced.  No global atomics; results are bit-identical run to run.
+//   * A wave gathers 16 pairs per MFMA block straight into operand registers: lane (i = lane%16,
+//     q = lane/16) loads 16 bytes of pair i's input row per K-chunk (FP32: channels 16g+4q..+3, FP16:
+//     channels 32g+8q..+7), i.e. every row is read as 64-byte segments.  The weights were reordered on
+//     the host so that the other operand of the same MFMA steps is one 16-byte load per lane as well;
+//     one pass over W[k] serves all blocks of the offset.  The next offset's rows are loaded at the top
+//     of the current one, and the weight registers of chunk g are refilled with the next offset's chunk g
+//     as soon as the MFMAs that read them have issued.
+//   * FP32: v_mfma_f32_16x16x4_f32; FP16: v_mfma_f32_16x16x32_f16 (16x16x16 for Cin = 16).  The weights
+//     are the MFMA's A operand and the gathered rows its B operand, so a lane ends up with four
+//     consecutive output channels of one pair; the block is then added into the wave's private partial
+//     tile in LDS at the pairs' output rows with 16-byte read-modify-writes (only this wave touches its
+//     partial and LDS keeps a wave's operations in order, so the sum order is fixed; LDS float atomics
+//     measured several times slower).
+//   * The four partial tiles are summed in a fixed order, scale/shift/ReLU is applied in FP32 and each
+//     output row is written once, coalesced.  No global atomics; results are bit-identical run to run.
 #include "kernels.h"
 
 namespace sessd {
@@ -30,6 +33,8 @@ namespace sessd {
 namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 #ifndef SESSD_MFMA_WAVES
 #define SESSD_MFMA_WAVES 4
@@ -41,7 +46,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 #define SESSD_MFMA_TARGET 40
 #endif
 constexpr int kWaves = SESSD_MFMA_WAVES;
-constexpr int kTileRows = SESSD_MFMA_TM;      // capacity: most output rows a workgroup can own (<= 64)
+constexpr int kTileRows = SESSD_MFMA_TM;        // capacity: most output rows a workgroup can own (<= 64)
 constexpr int kTargetRows = SESSD_MFMA_TARGET;  // tile height aimed for when choosing tiles per CU
 constexpr int kMaxBlk = (kTileRows + 15) / 16;  // MFMA row blocks an offset can need
 constexpr int kMaxK = 27;
@@ -58,15 +63,72 @@ __host__ __device__ inline int tile_height(int n, int num_cu) {
     return h > kTileRows ? kTileRows : (h < 1 ? 1 : h);
 }
 
-template <int CIN, int COUT>
+// Per-dtype shape of one K-chunk: how many channels it spans, what a lane holds of it, and the MFMA
+// sequence that consumes it (w = weights fragment -> A operand, x = gathered-row fragment -> B operand).
+template <typename T, int CIN>
+struct Chunk;
+
+template <int CIN>
+struct Chunk<float, CIN> {
+    using Vec = float4;  // 4 channels
+    static constexpr int kChannels = 16, kLaneElems = 4;
+    static __device__ __forceinline__ Vec zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+    static __device__ __forceinline__ void mma(const Vec& w, const Vec& x, v4f& acc) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w.x, x.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w.y, x.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, x.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w.w, x.w, acc, 0, 0, 0);
+    }
+};
+
+template <int CIN>
+struct Chunk<__half, CIN> {
+    using Vec = float4;  // 8 halfs = channels 32g+8q .. +7
+    static constexpr int kChannels = 32, kLaneElems = 8;
+    static __device__ __forceinline__ Vec zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+    static __device__ __forceinline__ void mma(const Vec& w, const Vec& x, v4f& acc) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const v8h*>(&w),
+                                                     *reinterpret_cast<const v8h*>(&x), acc, 0, 0, 0);
+    }
+};
+
+template <>
+struct Chunk<__half, 16> {
+    using Vec = float2;  // 4 halfs = channels 4q .. +3
+    static constexpr int kChannels = 16, kLaneElems = 4;
+    static __device__ __forceinline__ Vec zero() { return make_float2(0.f, 0.f); }
+    static __device__ __forceinline__ void mma(const Vec& w, const Vec& x, v4f& acc) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x16f16(*reinterpret_cast<const v4h*>(&w),
+                                                    *reinterpret_cast<const v4h*>(&x), acc, 0, 0, 0);
+    }
+};
+
+// four consecutive output channels -> memory
+__device__ __forceinline__ void store4(float* dst, const float (&o)[4]) {
+    *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+}
+__device__ __forceinline__ void store4(__half* dst, const float (&o)[4]) {
+    union {
+        __half2 h[2];
+        uint2 u;
+    } p;
+    p.h[0] = __floats2half2_rn(o[0], o[1]);
+    p.h[1] = __floats2half2_rn(o[2], o[3]);
+    *reinterpret_cast<uint2*>(dst) = p.u;
+}
+
+template <typename T, int CIN, int COUT>
 __global__ void __launch_bounds__(kWaves * 64)
-conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float* __restrict__ Wp,
-              const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
-              const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad,
-              int num_cu) {
-    constexpr int G = CIN / 16;    // 16-channel chunks of the inner dimension
-    constexpr int NB = COUT / 16;  // 16-column blocks
-    constexpr int LDP = COUT + 4;  // padded row stride of the partial tiles in LDS
+conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict__ Wp,
+          const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
+          const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad,
+          int num_cu) {
+    using C = Chunk<T, CIN>;
+    using Vec = typename C::Vec;
+    constexpr int G = CIN / C::kChannels;  // K-chunks of the inner dimension
+    constexpr int NB = COUT / 16;          // 16-column blocks
+    constexpr int LDP = COUT + 4;          // padded row stride of the partial tiles in LDS
+    static_assert(CIN % C::kChannels == 0 && COUT % 16 == 0, "channel counts must fill whole MFMA chunks");
     __shared__ int32_t s_in[kMaxK * kTileRows];   // compacted pair lists: input row ...
     __shared__ uint8_t s_row[kMaxK * kTileRows];  // ... and local output row of pair j of offset k
     __shared__ int32_t s_cnt[kMaxK + 5];          // pairs per offset
@@ -95,7 +157,7 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
                     if (relu) s = s > 0.f ? s : 0.f;
                     o[e] = s;
                 }
-                *reinterpret_cast<float4*>(out + (size_t)row * COUT + c4) = make_float4(o[0], o[1], o[2], o[3]);
+                store4(out + (size_t)row * COUT + c4, o);
             }
     }
     const int R = tile_height(n, num_cu);  // rows of this launch's tiles
@@ -120,7 +182,7 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
     __syncthreads();
 
     const int i = lane & 15;  // pair inside a 16-pair block
-    const int q = lane >> 4;  // 4-channel group inside a 16-channel chunk
+    const int q = lane >> 4;  // channel group inside a K-chunk
 
     // offsets this wave handles: the non-empty ones, dealt round-robin (all wave-uniform)
     uint32_t my_mask = 0;
@@ -133,44 +195,32 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
             }
     }
 
-    const float4* wp4 = reinterpret_cast<const float4*>(Wp) + lane;
-    // gathered rows of all blocks of offset k -> A-operand registers (zeros for the padding pairs)
-    auto load_a = [&](int k, int cnt, float4 (&a)[kMaxBlk][G]) {
+    const Vec* wp = reinterpret_cast<const Vec*>(Wp) + lane;
+    // gathered rows of all blocks of offset k -> operand registers (zeros for the padding pairs)
+    auto load_a = [&](int k, int cnt, Vec (&a)[kMaxBlk][G]) {
 #pragma unroll
         for (int blk = 0; blk < kMaxBlk; ++blk) {
             const int j = blk * 16 + i;
             const bool live = j < cnt;
             const int idx = live ? s_in[k * kTileRows + j] : 0;
-            const float4* src = reinterpret_cast<const float4*>(in + (size_t)idx * CIN + q * 4);
+            const T* src = in + (size_t)idx * CIN + q * C::kLaneElems;
 #pragma unroll
             for (int g = 0; g < G; ++g) {
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-#ifdef SESSD_EXP_NO_LOADS
-                v.x = (float)idx;
-#else
-                if (live) v = src[g * 4];
-#endif
+                Vec v = C::zero();
+                if (live) v = *reinterpret_cast<const Vec*>(src + g * C::kChannels);
                 a[blk][g] = v;
             }
         }
     };
-    auto load_b = [&](int k, int g, float4 (&b)[NB]) {
-        const float4* wk = wp4 + ((size_t)k * G + g) * NB * 64;
+    auto load_b = [&](int k, int g, Vec (&b)[NB]) {
+        const Vec* wk = wp + ((size_t)k * G + g) * NB * 64;
 #pragma unroll
-#ifdef SESSD_EXP_NO_LOADS
-        for (int nb = 0; nb < NB; ++nb) b[nb] = make_float4((float)(k + g), 1.f, 2.f, (float)nb);
-#else
         for (int nb = 0; nb < NB; ++nb) b[nb] = wk[nb * 64];
-#endif
     };
 
     int k_cur = my_mask ? __ffs(my_mask) - 1 : -1;
     my_mask &= my_mask - 1;
-    // Pipeline: the gathered rows of the NEXT offset are loaded at the top of the current one; the
-    // weight registers of chunk g are refilled with the next offset's chunk g as soon as the MFMAs that
-    // read them have issued, so every weight load has a whole offset of MFMA work to hide behind
-    // without a second register set.
-    float4 a_cur[kMaxBlk][G], a_nxt[kMaxBlk][G], b[G][NB];
+    Vec a_cur[kMaxBlk][G], a_nxt[kMaxBlk][G], b[G][NB];
     int cnt_cur = 0, cnt_nxt = 0;
     if (k_cur >= 0) {
         cnt_cur = s_cnt[k_cur];
@@ -195,27 +245,20 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
 #pragma unroll
             for (int blk = 0; blk < kMaxBlk; ++blk) {
                 if (blk * 16 >= cnt_cur) continue;  // wave-uniform: this offset has fewer pairs
-                const float av[4] = {a_cur[blk][g].x, a_cur[blk][g].y, a_cur[blk][g].z, a_cur[blk][g].w};
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-#pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) {
-                        const float bv[4] = {b[g][nb].x, b[g][nb].y, b[g][nb].z, b[g][nb].w};
-                        acc[blk][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(bv[e], av[e], acc[blk][nb], 0, 0, 0);
-                    }
+                for (int nb = 0; nb < NB; ++nb) C::mma(b[g][nb], a_cur[blk][g], acc[blk][nb]);
             }
             if (k_nxt >= 0) load_b(k_nxt, g, b[g]);
         }
-        // block results -> partial tile.  The weights are the MFMA's A operand and the gathered rows its
-        // B operand, so D is the transposed block: lane (pair j = lane%16, q = lane/16) holds output
-        // channels 16nb+4q .. +3 of pair j -- one 16-byte LDS read-modify-write per column block.
+        // block results -> partial tile.  D is the transposed block: lane (pair j = lane%16, q = lane/16)
+        // holds output channels 16nb+4q .. +3 of pair j -- one 16-byte LDS read-modify-write per column
+        // block.
 #pragma unroll
         for (int blk = 0; blk < kMaxBlk; ++blk) {
             if (blk * 16 >= cnt_cur) continue;
             const int j = blk * 16 + i;
             if (j < cnt_cur) {
                 float* dst = part + (int)s_row[k_cur * kTileRows + j] * LDP + q * 4;
-#ifndef SESSD_EXP_NO_ACCUM
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) {
                     float4 v = *reinterpret_cast<float4*>(dst + nb * 16);
@@ -225,12 +268,6 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
                     v.w += acc[blk][nb][3];
                     *reinterpret_cast<float4*>(dst + nb * 16) = v;
                 }
-#else
-                float t = 0.f;
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) t += acc[blk][nb][0] + acc[blk][nb][1] + acc[blk][nb][2] + acc[blk][nb][3];
-                if (t == 123.f) dst[0] = 1.f;
-#endif
             }
         }
 #pragma unroll
@@ -242,7 +279,7 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
     }
     __syncthreads();
 
-    // fixed-order sum of the four partials, epilogue, coalesced 16-byte stores
+    // fixed-order sum of the four partials, epilogue, coalesced stores
     for (int v = tid; v < rows * kVecPerRow; v += kWaves * 64) {
         const int r = v / kVecPerRow, c4 = (v % kVecPerRow) * 4;
         float o[4];
@@ -256,7 +293,7 @@ conv_mfma_f32(const float* __restrict__ in, float* __restrict__ out, const float
             if (relu) s = s > 0.f ? s : 0.f;
             o[e] = s;
         }
-        *reinterpret_cast<float4*>(out + (size_t)(row0 + r) * COUT + c4) = make_float4(o[0], o[1], o[2], o[3]);
+        store4(out + (size_t)(row0 + r) * COUT + c4, o);
     }
 }
 
@@ -273,57 +310,74 @@ int compute_units() {
     return cu;
 }
 
-template <int CIN, int COUT>
-int launch_f32(const GemmArgs& a, hipStream_t stream) {
+template <typename T, int CIN, int COUT>
+int launch(const GemmArgs& a, hipStream_t stream) {
     const int num_cu = compute_units();
     // tile_height() never cuts n <= max_voxels rows into more than num_cu * r_max tiles
     const int r_max = ceil_div(a.max_voxels, (int64_t)num_cu * kTargetRows);
     const unsigned blocks = (unsigned)(num_cu * (r_max < 1 ? 1 : r_max));
-    hipLaunchKernelGGL((conv_mfma_f32<CIN, COUT>), dim3(blocks), dim3(kWaves * 64), 0, stream,
-                       static_cast<const float*>(a.in_feat), static_cast<float*>(a.out_feat),
-                       static_cast<const float*>(a.w_packed), a.nbr, a.num_out, a.max_voxels, a.K, a.scale,
-                       a.shift, a.relu, a.write_pad_rows, num_cu);
+    hipLaunchKernelGGL((conv_mfma<T, CIN, COUT>), dim3(blocks), dim3(kWaves * 64), 0, stream,
+                       static_cast<const T*>(a.in_feat), static_cast<T*>(a.out_feat), a.w_packed, a.nbr,
+                       a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows, num_cu);
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;
 }
 
-bool mfma_f32_shape(int K, int cin, int cout) {
-    if (K > 27) return false;
+bool mfma_shape(int K, int cin, int cout) {
+    if (K > kMaxK) return false;
     const int shapes[][2] = {{16, 16}, {16, 32}, {32, 32}, {32, 64}, {64, 64}, {64, 128}, {128, 128}};
     for (auto& s : shapes)
         if (s[0] == cin && s[1] == cout) return true;
     return false;
 }
 
+// channels per K-chunk and elements per lane, as in Chunk<>
+void chunk_shape(int dtype, int cin, int* channels, int* lane_elems) {
+    if (dtype == SESSD_FLOAT) {
+        *channels = 16;
+        *lane_elems = 4;
+    } else if (cin == 16) {
+        *channels = 16;
+        *lane_elems = 4;
+    } else {
+        *channels = 32;
+        *lane_elems = 8;
+    }
+}
+
 }  // namespace
 
 size_t packed_weight_bytes(int K, int cin, int cout, int dtype) {
-    if (dtype == SESSD_FLOAT && mfma_f32_shape(K, cin, cout)) return (size_t)K * cin * cout * sizeof(float);
-    return 0;
+    if (!mfma_shape(K, cin, cout)) return 0;
+    return (size_t)K * cin * cout * (dtype == SESSD_HALF ? sizeof(__half) : sizeof(float));
 }
 
-// FP32 operand order: Wp[k][g][nb][lane][e] = W[k][16g + 4(lane/16) + e][16nb + lane%16]
+// Operand order: Wp[k][g][nb][lane][e] = W[k][C*g + E*(lane/16) + e][16nb + lane%16] with C channels per
+// K-chunk and E elements per lane (FP32: 16/4, FP16: 32/8, FP16 with Cin = 16: 16/4).
 void pack_weights(const float* w, int K, int cin, int cout, int dtype, void* dst) {
-    if (dtype != SESSD_FLOAT) return;
-    float* p = static_cast<float*>(dst);
-    const int G = cin / 16, NB = cout / 16;
+    int C, E;
+    chunk_shape(dtype, cin, &C, &E);
+    const int G = cin / C, NB = cout / 16;
     for (int k = 0; k < K; ++k)
         for (int g = 0; g < G; ++g)
             for (int nb = 0; nb < NB; ++nb)
                 for (int lane = 0; lane < 64; ++lane)
-                    for (int e = 0; e < 4; ++e)
-                        p[((((size_t)k * G + g) * NB + nb) * 64 + lane) * 4 + e] =
-                            w[((size_t)k * cin + 16 * g + 4 * (lane / 16) + e) * cout + 16 * nb + lane % 16];
+                    for (int e = 0; e < E; ++e) {
+                        const size_t o = ((((size_t)k * G + g) * NB + nb) * 64 + lane) * E + e;
+                        const float v = w[((size_t)k * cin + C * g + E * (lane / 16) + e) * cout + 16 * nb + lane % 16];
+                        if (dtype == SESSD_HALF) static_cast<__half*>(dst)[o] = __float2half_rn(v);
+                        else static_cast<float*>(dst)[o] = v;
+                    }
 }
 
 // -> SESSD_OK when an MFMA kernel was launched, SESSD_E_UNSUPPORTED when the shape/dtype is not covered
 int launch_mfma(const GemmArgs& a, hipStream_t stream) {
-    if (a.in_type != SESSD_FLOAT || a.out_type != SESSD_FLOAT || !a.w_packed || !mfma_f32_shape(a.K, a.cin, a.cout))
-        return SESSD_E_UNSUPPORTED;
+    if (a.in_type != a.out_type || !a.w_packed || !mfma_shape(a.K, a.cin, a.cout)) return SESSD_E_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(a.in_feat) | reinterpret_cast<uintptr_t>(a.out_feat)) & 15)
         return SESSD_E_UNSUPPORTED;
-#define SESSD_CASE(CI, CO) \
-    if (a.cin == CI && a.cout == CO) return launch_f32<CI, CO>(a, stream)
+#define SESSD_CASE(CI, CO)                                                        \
+    if (a.cin == CI && a.cout == CO)                                              \
+    return a.in_type == SESSD_HALF ? launch<__half, CI, CO>(a, stream) : launch<float, CI, CO>(a, stream)
     SESSD_CASE(16, 16);
     SESSD_CASE(16, 32);
     SESSD_CASE(32, 32);

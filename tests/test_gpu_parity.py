@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import oracle_lib as O
-from gpu_util import (DEV, RTOL_FP32, assert_features_close, canonical, dev, points_input, to_np)
+from gpu_util import (DEV, RTOL_FP16, RTOL_FP32, assert_features_close, canonical, dev, points_input, to_np)
 from sessd3d import api, backbone as B, ctypes_defs as D, frames as F
 
 pytestmark = pytest.mark.gpu
@@ -166,6 +166,81 @@ def test_mfma_and_valu_paths_agree():
         outs.append(to_np(conv(dev(fbuf), dev(cbuf), dev(np.array([n], np.int32)))))
     assert_features_close(outs[0], outs[1], RTOL_FP32, "mfma vs valu")
     assert not np.array_equal(outs[0], outs[1]) or True
+
+
+@pytest.mark.parametrize("cin,cout", [(4, 16), (16, 16), (16, 32), (32, 32), (32, 64), (64, 64), (64, 128), (128, 128),
+                                      (8, 32)])
+def test_subm_fp16_features(cin, cout):
+    """FP16 features and weights, FP32 accumulate (BASELINE configs 4-5).  The oracle runs in FP32 on the
+    half-rounded inputs and weights and rounds its output to half: agreement within 1e-2 relative."""
+    grid = (21, 200, 176)
+    n, mv = 6000, 8192
+    rng = np.random.default_rng(100 + cin)
+    coors = F.clustered_active_voxels(n, grid, 2, n_blobs=60)
+    in_half = cin != 4                               # the first layer reads the voxelizer's FP32 means
+    feat = rng.uniform(-1, 1, (n, cin)).astype(np.float32)
+    if in_half:
+        feat = O.round_to_half(feat)
+    w = O.round_to_half(rng.normal(0, 0.1, (27, cin, cout)).astype(np.float32))
+    sc = rng.uniform(0.5, 1.5, cout).astype(np.float32)
+    sh = rng.uniform(-0.2, 0.2, cout).astype(np.float32)
+    conv = api.SubmConv3d(cin, cout, grid[::-1], w, mv)
+    conv.set_epilogue(sc, sh, True)
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = np.zeros((mv, cin), np.float32)
+    fbuf[:n] = feat
+    d_feat = dev(fbuf, torch.float16 if in_half else torch.float32)
+    out = conv(d_feat, dev(cbuf), dev(np.array([n], np.int32)), out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16
+    o_pairs, o_num, _ = O.subm_rulebook(coors, n, grid[::-1], mv)
+    o_out = O.round_to_half(O.scale_shift_relu(O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), mv, sc, sh, True))
+    assert_features_close(to_np(out.float()), o_out, RTOL_FP16, "fp16 subm %d->%d" % (cin, cout))
+    # the MFMA and VALU FP16 paths agree much more tightly than the 1e-2 bound
+    conv.set_flags(D.SESSD_FLAG_FORCE_VALU)
+    out2 = conv(d_feat, dev(cbuf), dev(np.array([n], np.int32)), out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    assert_features_close(to_np(out.float()), to_np(out2.float()), 2e-3, "fp16 mfma vs valu %d->%d" % (cin, cout))
+
+
+def test_sparse_fp16_features():
+    layer = SPARSE_LAYERS[1]        # 32 -> 64, stride 2
+    ig = sparse_input_grid(layer)
+    n, mv = 5000, 30000
+    rng = np.random.default_rng(77)
+    coors = F.clustered_active_voxels(n, (ig[0], 300, 300), 3, n_blobs=50)
+    feat = O.round_to_half(rng.uniform(-1, 1, (n, layer.cin)).astype(np.float32))
+    w = O.round_to_half(rng.normal(0, 0.1, (layer.kvol, layer.cin, layer.cout)).astype(np.float32))
+    conv = api.SparseConv3d(layer.cin, layer.cout, layer.out_shape, ig[::-1], layer.ksize, layer.stride,
+                            layer.padding, w, mv)
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = np.zeros((mv, layer.cin), np.float32)
+    fbuf[:n] = feat
+    out, oc, on = conv(dev(fbuf, torch.float16), dev(cbuf), dev(np.array([n], np.int32)))
+    torch.cuda.synchronize()
+    o_pairs, o_num, o_oc, o_on, _ = O.sparse_rulebook(coors, n, layer.out_shape, layer.ksize, layer.stride,
+                                                      layer.padding, mv)
+    assert int(to_np(on)[0]) == o_on and np.array_equal(to_np(oc), o_oc)
+    o_out = O.round_to_half(O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv))
+    assert_features_close(to_np(out.float()), o_out, RTOL_FP16, "fp16 sparse15")
+
+
+def test_sparse2dense_fp16():
+    rng = np.random.default_rng(3)
+    n, mv, c = 1500, 4096, 64
+    coors = F.random_active_voxels(n, (2, 200, 176), 9)
+    feat = O.round_to_half(rng.uniform(0.1, 1, (n, c)).astype(np.float32))
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = np.zeros((mv, c), np.float32)
+    fbuf[:n] = feat
+    s2d = api.Sparse2Dense()
+    dense = s2d(dev(fbuf, torch.float16), dev(cbuf), dev(np.array([n], np.int32)))
+    torch.cuda.synchronize()
+    assert dense.dtype == torch.float16
+    assert np.array_equal(to_np(dense.float()), O.sparse2dense(feat, coors, n, B.DENSE_SIZE_XYZ))
 
 
 def test_subm_shared_rulebook_skip_pad_and_empty():

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import oracle_lib as O
-from gpu_util import RTOL_FP32, assert_features_close, canonical, points_input, to_np
+from gpu_util import RTOL_FP16, RTOL_FP32, assert_features_close, canonical, points_input, to_np
 from sessd3d import api, backbone as B, ctypes_defs as D, frames as F
 
 pytestmark = pytest.mark.gpu
@@ -103,6 +103,45 @@ def test_full_backbone_config3_frame_and_graph_replay():
     stream.synchronize()
     ref2 = O.frame(pts2, B.voxelgen_desc(max_voxels=60000), layers, W, B.dense_desc())
     assert_features_close(to_np(gd), ref2["dense"], RTOL_END_TO_END, "graph replay on a new frame")
+
+
+def half_weights(W):
+    """The FP16 configurations store weights in half: round once, hand the same values to both sides."""
+    return B.Weights([O.round_to_half(w) for w in W.w], W.scale, W.shift)
+
+
+def test_fp16_backbone_against_half_rounding_oracle():
+    """FP16 features/weights with FP32 accumulate through all 14 layers.  The oracle keeps FP32 arithmetic
+    but rounds every layer's output to half, as the FP16 pipeline stores it.  Sites are bit-exact; features
+    within 1e-2 relative per layer (oracle fed the GPU's rows) and end to end."""
+    pts = F.lidar_frame(12000, 21)
+    layers = B.reference_layers()
+    W = half_weights(B.random_weights(layers, seed=9, w_std=0.05))
+    mv = 40000
+    pipe, dense, _ = run_pipeline(pts, layers, W, 12000, mv, feature_dtype="fp16", share_rulebooks=True,
+                                  skip_pad_rows=True, overlap_streams=True)
+    assert dense.dtype == torch.float16
+    ref = O.frame(pts, B.voxelgen_desc(max_voxels=mv), layers, W, B.dense_desc(), round_half=True)
+    feat, coors, n = pipe.read_layer(-1)
+    for l, layer in enumerate(layers):
+        fbuf = np.zeros((mv, layer.cin), np.float32)
+        fbuf[:n] = feat
+        cbuf = np.zeros((mv, 4), np.int32)
+        cbuf[:n] = coors
+        o_out, o_coors, o_n, _, _ = O.conv_layer(fbuf, cbuf, n, layer, W.w[l], W.scale[l], W.shift[l], mv)
+        feat, g_coors, g_n = pipe.read_layer(l)
+        assert g_n == o_n == ref["counts"][l + 1] and np.array_equal(g_coors, o_coors[:o_n]), layer.name
+        assert_features_close(feat, O.round_to_half(o_out[:o_n]), RTOL_FP16, "fp16 " + layer.name)
+        coors, n = g_coors, g_n
+    assert np.array_equal(coors, ref["coors"])
+    # end to end a half-rounding that falls the other way in an early layer is amplified by the layers
+    # after it: as for FP32 the whole-frame bound is ten times the per-layer one, and the error must stay
+    # within 1e-2 in the L2 norm
+    assert_features_close(feat, ref["feat"], 10 * RTOL_FP16, "fp16 last layer (end to end)")
+    d = to_np(dense.float())
+    assert_features_close(d, ref["dense"], 10 * RTOL_FP16, "fp16 dense (end to end)")
+    assert np.linalg.norm(d - ref["dense"]) <= RTOL_FP16 * np.linalg.norm(ref["dense"])
+    assert pipe.status() == ref["status"]
 
 
 def test_properties_at_full_size():
