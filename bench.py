@@ -46,13 +46,14 @@ def profiled_traffic(kernel, dtype):
     return None
 
 
-def cpu_baseline(pts, layers, W, max_voxels, budget_s=20.0):
+def cpu_baseline(pts, layers, W, max_voxels, voxel_cap, budget_s=20.0):
     """The scalar CPU port (the parity oracle) on the same frame, one thread, a bounded number of frames."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_lib as O
     from sessd3d import backbone as B
-    vg = B.voxelgen_desc(max_voxels=max_voxels)
-    dd = B.dense_desc()
+    # (the oracle uses one capacity for every tensor; the voxelizer's cap equals it in the headline config)
+    vg = B.voxelgen_desc(max_voxels=max_voxels if voxel_cap >= max_voxels else voxel_cap)
+    dd = B.dense_desc(channel=layers[-1].cout)
     times = []
     t_start = time.perf_counter()
     O.frame(pts, vg, layers, W, dd)          # warm-up (allocates the dense index grids)
@@ -72,10 +73,14 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--points", type=int, default=20000)
+    ap.add_argument("--config", type=int, default=3, choices=[3, 4, 5],
+                    help="BASELINE configuration: 3 = 20k points FP32 (headline), 4 = 60k points, voxel cap 40k, FP16, "
+                         "5 = 150k points over 360 degrees, voxel cap 60k, doubled channel widths, FP16")
+    ap.add_argument("--points", type=int, default=None)
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--dtype", default="fp32", choices=["fp32", "fp16"])
-    ap.add_argument("--max-voxels", type=int, default=60000)
+    ap.add_argument("--dtype", default=None, choices=["fp32", "fp16"])
+    ap.add_argument("--max-voxels", type=int, default=None, help="rows of the conv layers' tensors")
+    ap.add_argument("--voxel-cap", type=int, default=None, help="the voxelizer's max_voxels")
     ap.add_argument("--no-graph", action="store_true", help="launch kernels directly instead of replaying a hipGraph")
     ap.add_argument("--no-share", action="store_true", help="every SubM layer rebuilds its rulebook (as the reference does)")
     ap.add_argument("--pad-rows", action="store_true", help="write rows >= voxel_num of every tensor (reference behaviour)")
@@ -98,13 +103,21 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
-    layers = B.reference_layers()
+    preset = {3: dict(points=20000, dtype="fp32", max_voxels=60000, voxel_cap=60000, width=1, full=False),
+              4: dict(points=60000, dtype="fp16", max_voxels=100000, voxel_cap=40000, width=1, full=False),
+              5: dict(points=150000, dtype="fp16", max_voxels=200000, voxel_cap=60000, width=2, full=True)}[args.config]
+    args.points = args.points or preset["points"]
+    args.dtype = args.dtype or preset["dtype"]
+    args.max_voxels = args.max_voxels or preset["max_voxels"]
+    args.voxel_cap = args.voxel_cap or preset["voxel_cap"]
+    layers = B.reference_layers(width_mult=preset["width"])
     W = B.random_weights(layers, seed=1, w_std=0.05 if args.dtype == "fp16" else 0.1)
-    pts = F.lidar_frame(args.points, args.seed)
+    pts = F.lidar_frame(args.points, args.seed, full_circle=preset["full"])
     max_points = args.points
     pipe = api.Pipeline(layers, W, max_points, args.max_voxels, feature_dtype=args.dtype,
                         share_rulebooks=not args.no_share, skip_pad_rows=not args.pad_rows,
-                        use_graph=not args.no_graph, overlap_streams=not args.no_overlap)
+                        use_graph=not args.no_graph, overlap_streams=not args.no_overlap, voxel_cap=args.voxel_cap,
+                        dense_size_xyz=B.DENSE_SIZE_XYZ)
     points = torch.as_tensor(pts).to(dev)
     size = torch.tensor([len(pts)], dtype=torch.int32, device=dev)
     dense = pipe.new_dense(dev)
@@ -159,7 +172,8 @@ def main():
                           "gemm_tflops": round(fl / (seg[2 + 2 * l] * 1e-3) / 1e12, 3) if seg[2 + 2 * l] > 0 else None,
                           "gemm_gbs": round(by / (seg[2 + 2 * l] * 1e-3) / 1e9, 1) if seg[2 + 2 * l] > 0 else None})
     # dominant kernel: the gather-GEMM instantiation for 64 -> 64 channels (six launches per frame)
-    dom = [l for l, layer in enumerate(layers) if layer.cin == 64 and layer.cout == 64]
+    dom_c = 64 * preset["width"]
+    dom = [l for l, layer in enumerate(layers) if layer.cin == dom_c and layer.cout == dom_c]
     dom_flops = sum(layer_work(layers[l], *stats[l], esize)[0] for l in dom) / len(dom)
     dom_bytes = sum(layer_work(layers[l], *stats[l], esize)[1] for l in dom) / len(dom)
     dom_ms = sum(seg[2 + 2 * l] for l in dom) / len(dom)
@@ -174,8 +188,9 @@ def main():
         ach = dom_bytes / (dom_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None}
-    roof["traffic"] = profiled_traffic("conv_mfma_%s<64, 64>" % ("f16" if args.dtype == "fp16" else "f32"), args.dtype)
-    roof.update({"kernel": "gather-GEMM 64->64 (%s)" % args.dtype, "launches_per_frame": len(dom),
+    kname = "conv_mfma<%s, %d, %d>" % ("__half" if args.dtype == "fp16" else "float", dom_c, dom_c)
+    roof["traffic"] = profiled_traffic(kname, args.dtype) if args.config == 3 else None
+    roof.update({"kernel": "gather-GEMM %d->%d (%s)" % (dom_c, dom_c, args.dtype), "launches_per_frame": len(dom),
                  "avg_launch_us": round(dom_ms * 1e3, 2), "algorithmic_flops_per_launch": dom_flops,
                  "algorithmic_bytes_per_launch": dom_bytes})
     # whole-frame algorithmic traffic: voxelizer + conv layers + sparse2dense (dense tensor written once)
@@ -187,10 +202,11 @@ def main():
         "value": round(ms_per_frame, 4), "unit": "ms/frame", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_frame, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16" if args.dtype == "fp16" else "f32", "data": "synthetic",
-        "config": {"workload": "config 3: %d-point seeded synthetic LiDAR frame (seed %d), %d voxels, reference 14-layer "
-                               "SpMiddleFHD backbone (10 SubM + 4 SparseConv, BN folded + ReLU), sparse2Dense to 128x200x176"
-                               % (len(pts), args.seed, n_vox),
-                   "max_voxels": args.max_voxels, "graph": not args.no_graph, "overlap_streams": not args.no_overlap, "share_rulebooks": not args.no_share,
+        "config": {"workload": "config %d: %d-point seeded synthetic LiDAR frame (seed %d), %d voxels, reference 14-layer "
+                               "SpMiddleFHD backbone (10 SubM + 4 SparseConv, channel widths x%d, BN folded + ReLU), "
+                               "sparse2Dense to %dx200x176"
+                               % (args.config, len(pts), args.seed, n_vox, preset["width"], layers[-1].cout * 2),
+                   "max_voxels": args.max_voxels, "voxel_cap": args.voxel_cap, "graph": not args.no_graph, "overlap_streams": not args.no_overlap, "share_rulebooks": not args.no_share,
                    "pad_rows": args.pad_rows, "n_layers": len(layers)},
         "roofline": roof,
         "frame": {"frames_per_s": round(1e3 / ms_per_frame, 1), "algorithmic_gflop": round(tot_flops / 1e9, 3),
@@ -210,7 +226,7 @@ def main():
         torch.cuda.synchronize()
         out["calibration"] = {"copy_mib": args.calibrate_mb, "repeats": 3}
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(pts, layers, W, args.max_voxels)
+        out["cpu_baseline"] = cpu_baseline(pts, layers, W, args.max_voxels, args.voxel_cap)
     print(json.dumps(out))
 
 

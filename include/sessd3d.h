@@ -322,6 +322,8 @@ typedef struct sessd_pipeline_desc {
     int32_t share_rulebooks;     /* consecutive SubM layers on one coors tensor build it once */
     int32_t flags;               /* SESSD_FLAG_* applied to every layer */
     int32_t use_graph;           /* replay the enqueue sequence from a captured hipGraph */
+    int32_t layer_max_voxels;    /* rows of the conv layers' tensors; 0 = voxelgen.max_voxels.  May exceed the
+                                    voxelizer's cap: strided layers can produce more sites than they get */
     int32_t overlap_streams;     /* run the coordinate chain (voxelizer + rulebook builds) on a second
                                     stream owned by the pipeline, overlapping the GEMMs of earlier layers */
 } sessd_pipeline_desc;

@@ -183,7 +183,11 @@ static int build_pipeline(const sessd_pipeline_desc& d, Pipeline* P) {
         return fail(SESSD_E_UNSUPPORTED, "pipeline: feature_dtype must be FP32 or FP16");
     if (d.max_points <= 0 || d.point_features < 4) return fail(SESSD_E_INVALID, "pipeline: bad points shape");
     P->desc = d;
-    const int V = d.voxelgen.max_voxels;
+    // rows of every conv-layer tensor; the voxelizer's own cap (voxelgen.max_voxels) may be lower: strided
+    // layers can produce more sites than they are given
+    const int V = d.layer_max_voxels > 0 ? d.layer_max_voxels : d.voxelgen.max_voxels;
+    if (V < d.voxelgen.max_voxels) return fail(SESSD_E_INVALID, "pipeline: layer_max_voxels below the voxelizer's cap");
+    const int VG = d.voxelgen.max_voxels;
     P->max_voxels = V;
     const int ft = d.feature_dtype;
     size_t total = 0;
@@ -194,8 +198,8 @@ static int build_pipeline(const sessd_pipeline_desc& d, Pipeline* P) {
     vg->flags_ = d.flags;
     P->vg_in[0] = make_desc({1, d.max_points, d.point_features}, SESSD_FLOAT);
     P->vg_in[1] = make_desc({1}, SESSD_INT32);
-    P->vg_out[0] = make_desc({1, V, 4}, SESSD_FLOAT);
-    P->vg_out[1] = make_desc({1, V, 4}, SESSD_INT32);
+    P->vg_out[0] = make_desc({1, VG, 4}, SESSD_FLOAT);
+    P->vg_out[1] = make_desc({1, VG, 4}, SESSD_INT32);
     P->vg_out[2] = make_desc({1}, SESSD_INT32);
     SESSD_TRY(vg->configurePlugin(P->vg_in, 2, P->vg_out, 3));
     SESSD_TRY(P->vg_ws.alloc(vg->getWorkspaceSize(P->vg_in, 2, P->vg_out, 3)));

@@ -349,10 +349,13 @@ class Pipeline:
     def __init__(self, layers, weights: B.Weights, max_points, max_voxels=B.MAX_VOXELS, point_features=4,
                  feature_dtype="fp32", relu=True, share_rulebooks=True, skip_pad_rows=False, use_graph=False,
                  dense_size_xyz=B.DENSE_SIZE_XYZ, max_pts_per_voxel=B.MAX_NUM_POINTS_PER_VOXEL,
-                 use_epilogue=True, overlap_streams=False):
+                 use_epilogue=True, overlap_streams=False, voxel_cap=None):
+        """max_voxels = rows of every conv-layer tensor; voxel_cap (default: max_voxels) = the voxelizer's
+        own limit."""
         torch = _torch()
         self.layers = list(layers)
         self.max_points, self.max_voxels = max_points, max_voxels
+        self.voxel_cap = voxel_cap or max_voxels
         self.dtype = torch.float16 if feature_dtype in ("fp16", "half", torch.float16) else torch.float32
         n = len(self.layers)
         self._specs = B.layer_specs(self.layers)
@@ -362,7 +365,8 @@ class Pipeline:
         FP = C.POINTER(C.c_float)
         arr = lambda xs: (FP * max(n, 1))(*[x.ctypes.data_as(FP) for x in xs])  # noqa: E731
         d = D.PipelineDesc()
-        d.voxelgen = B.voxelgen_desc(max_voxels, max_pts_per_voxel)
+        d.voxelgen = B.voxelgen_desc(voxel_cap or max_voxels, max_pts_per_voxel)
+        d.layer_max_voxels = max_voxels
         d.max_points, d.point_features, d.n_layers = max_points, point_features, n
         d.layers = self._specs
         d.weights = arr(self._w)
@@ -404,8 +408,9 @@ class Pipeline:
         _hip_d2h(num, n)
         cnt = int(num[0])
         es = 4 if (layer < 0 or self.dtype == torch.float32) else 2
-        feat = np.zeros((self.max_voxels, ch), np.float32 if es == 4 else np.float16)
-        coors = np.zeros((self.max_voxels, 4), np.int32)
+        rows = self.voxel_cap if layer < 0 else self.max_voxels
+        feat = np.zeros((rows, ch), np.float32 if es == 4 else np.float16)
+        coors = np.zeros((rows, 4), np.int32)
         _hip_d2h(feat, f)
         _hip_d2h(coors, c)
         return feat[:cnt].astype(np.float32), coors[:cnt], cnt

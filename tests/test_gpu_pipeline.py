@@ -166,3 +166,35 @@ def test_properties_at_full_size():
     vfeat, vcoors, vn = pipe.read_layer(-1)
     o = O.voxelize(pts, B.POINT_CLOUD_RANGE, B.VOXEL_SIZE, 5, 60000)
     assert vn == o[2] and np.array_equal(vcoors, o[1][:vn]) and np.array_equal(vfeat.view(np.uint32), o[0][:vn].view(np.uint32))
+
+
+def test_stress_configuration_properties():
+    """BASELINE config 5: 150 000 points over 360 degrees (cropped to range), voxel cap 60 000, doubled
+    channel widths, FP16 features.  Too heavy for the scalar oracle's conv layers, so: the voxelizer part
+    is compared with the oracle exactly (the cap binds -> overflow flag), the rest through properties."""
+    pts = F.lidar_frame(150000, 5, full_circle=True)
+    layers = B.reference_layers(width_mult=2)
+    W = half_weights(B.random_weights(layers, seed=4, w_std=0.03))
+    pipe, dense, (p, n, stream) = run_pipeline(pts, layers, W, 150000, 200000, feature_dtype="fp16",
+                                               skip_pad_rows=True, overlap_streams=True, use_graph=True,
+                                               voxel_cap=60000)
+    assert tuple(dense.shape) == (256, 200, 176)
+    first = to_np(dense).copy()
+    for _ in range(2):                                               # graph replays are bit identical
+        with torch.cuda.stream(stream):
+            pipe.enqueue(p, n, dense, stream)
+        stream.synchronize()
+        assert np.array_equal(to_np(dense), first)
+    vfeat, vcoors, vn = pipe.read_layer(-1)
+    o = O.voxelize(pts, B.POINT_CLOUD_RANGE, B.VOXEL_SIZE, 5, 60000)
+    assert vn == o[2] == 60000 and o[4] & D.SESSD_STATUS_VOXEL_OVERFLOW
+    assert np.array_equal(vcoors, o[1][:vn]) and np.array_equal(vfeat.view(np.uint32), o[0][:vn].view(np.uint32))
+    assert pipe.status() & D.SESSD_STATUS_VOXEL_OVERFLOW
+    counts = [pipe.layer_stats(l)[0] for l in range(len(layers))]
+    assert counts[0] == counts[1] == 60000 and max(counts) <= 200000
+    assert counts[2] > 60000                                         # the first strided layer grows the set
+    feat, coors, cnt = pipe.read_layer(len(layers) - 1)
+    assert cnt == counts[-1] and len(np.unique(coors[:, 1:] @ np.array([200 * 176, 176, 1]))) == cnt
+    back = first.reshape(128, 2, 200, 176)[:, coors[:, 1], coors[:, 2], coors[:, 3]].T
+    assert np.array_equal(back.astype(np.float32), feat)
+    assert np.isfinite(first.astype(np.float32)).all()
