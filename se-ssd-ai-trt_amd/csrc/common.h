@@ -139,10 +139,12 @@ struct FillRegion {
     uint32_t value;
 };
 struct FillArgs {
-    FillRegion r[6];
+    static constexpr int kMaxRegions = 16;
+    FillRegion r[kMaxRegions];
     int n = 0;
+    bool full() const { return n >= kMaxRegions; }
     void add(void* p, uint64_t words, uint32_t value) {
-        if (!p || !words) return;
+        if (!p || !words || n >= kMaxRegions) return;
         r[n].ptr = static_cast<uint32_t*>(p);
         r[n].words = words;
         r[n].value = value;

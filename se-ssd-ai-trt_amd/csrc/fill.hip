@@ -23,7 +23,7 @@ int fail(int code, const char* fmt, ...) {
 
 const char* last_error_cstr() { return g_last_error.c_str(); }
 
-// One launch clears up to six regions: blockIdx.y picks the region, blockIdx.x strides over it with
+// One launch clears up to FillArgs::kMaxRegions regions: blockIdx.y picks the region, blockIdx.x strides over it with
 // 16-byte stores (pure write stream, HBM-bound).
 __global__ void __launch_bounds__(256) fill_kernel(FillArgs a) {
     const FillRegion r = a.r[blockIdx.y];

@@ -69,8 +69,8 @@ struct Pipeline {
 
     // two-stream schedule: coordinate chain (voxelizer + rulebook builds) on `aux`, feature chain on the
     // caller's stream; ev_build[l] = "rulebook of layer l is ready"
-    hipStream_t aux = nullptr;
-    hipEvent_t ev_start = nullptr, ev_vg = nullptr;
+    hipStream_t aux = nullptr, aux_fill = nullptr;
+    hipEvent_t ev_start = nullptr, ev_vg = nullptr, ev_fill = nullptr;
     std::vector<hipEvent_t> ev_build;
 
     // profiling: one event per segment boundary (see sessd_pipeline_enqueue_timed)
@@ -85,7 +85,9 @@ struct Pipeline {
             if (e) (void)hipEventDestroy(e);
         if (ev_start) (void)hipEventDestroy(ev_start);
         if (ev_vg) (void)hipEventDestroy(ev_vg);
+        if (ev_fill) (void)hipEventDestroy(ev_fill);
         if (aux) (void)hipStreamDestroy(aux);
+        if (aux_fill) (void)hipStreamDestroy(aux_fill);
     }
 
     // The rulebooks depend only on coordinates, the GEMMs on rulebooks + features.  The coordinate chain
@@ -95,20 +97,42 @@ struct Pipeline {
     int enqueueOverlapped(const void* points, const void* points_size, void* dense, hipStream_t stream) {
         SESSD_HIP_TRY(hipEventRecord(ev_start, stream));
         SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_start, 0));
+        SESSD_HIP_TRY(hipStreamWaitEvent(aux_fill, ev_start, 0));
+        // every clear of the frame (hash tables, neighbour tables, status words, the dense tensor) has no
+        // input: they run batched on a third stream while the voxelizer works
+        {
+            FillArgs f;
+            auto flush = [&]() -> int {
+                const int rc = launch_fill(f, aux_fill);
+                f = FillArgs();
+                return rc;
+            };
+            for (auto& st : stages) {
+                if (!st->ws.p) continue;
+                if (f.n + 4 > FillArgs::kMaxRegions) SESSD_TRY(flush());
+                if (st->subm) st->subm->collectFill(st->ws.p, f);
+                else st->sparse->collectFill(st->ws.p, static_cast<int32_t*>(st->coors.p), f);
+            }
+            if (f.n + 2 > FillArgs::kMaxRegions) SESSD_TRY(flush());
+            s2d->collectFill(dense, s2d_ws.p, f);
+            SESSD_TRY(flush());
+            SESSD_HIP_TRY(hipEventRecord(ev_fill, aux_fill));
+        }
         const void* vin[2] = {points, points_size};
         void* vout[3] = {vg_voxels.p, vg_coors.p, vg_num.p};
         SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, aux));
         SESSD_HIP_TRY(hipEventRecord(ev_vg, aux));
+        SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_fill, 0));
         const int32_t* coors = static_cast<const int32_t*>(vg_coors.p);
         const int32_t* num = static_cast<const int32_t*>(vg_num.p);
         for (size_t l = 0; l < stages.size(); ++l) {
             ConvStage& st = *stages[l];
             if (st.subm) {
                 if (st.rulebook_from >= 0) continue;
-                SESSD_TRY(st.subm->enqueueBuild(coors, num, st.ws.p, aux));
+                SESSD_TRY(st.subm->enqueueBuild(coors, num, st.ws.p, aux, true));
             } else {
                 SESSD_TRY(st.sparse->enqueueBuild(coors, num, static_cast<int32_t*>(st.coors.p),
-                                                  static_cast<int32_t*>(st.num.p), st.ws.p, aux));
+                                                  static_cast<int32_t*>(st.num.p), st.ws.p, aux, true));
                 coors = static_cast<const int32_t*>(st.coors.p);
                 num = static_cast<const int32_t*>(st.num.p);
             }
@@ -137,9 +161,10 @@ struct Pipeline {
         }
         // every event of `aux` has been waited on by now (the last build is the last aux operation)
         if (stages.empty()) SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_vg, 0));
+        SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_fill, 0));
         const void* din[3] = {feat, coors, num};
         void* dout[1] = {dense};
-        return s2d->enqueue(s2d_in, s2d_out, din, dout, s2d_ws.p, stream);
+        return s2d->enqueue(s2d_in, s2d_out, din, dout, s2d_ws.p, stream, true);
     }
 
     int enqueueDirect(const void* points, const void* points_size, void* dense, hipStream_t stream) {
@@ -304,6 +329,8 @@ static int build_pipeline(const sessd_pipeline_desc& d, Pipeline* P) {
     P->device_bytes = total;
     if (d.overlap_streams) {
         SESSD_HIP_TRY(hipStreamCreateWithFlags(&P->aux, hipStreamNonBlocking));
+        SESSD_HIP_TRY(hipStreamCreateWithFlags(&P->aux_fill, hipStreamNonBlocking));
+        SESSD_HIP_TRY(hipEventCreateWithFlags(&P->ev_fill, hipEventDisableTiming));
         SESSD_HIP_TRY(hipEventCreateWithFlags(&P->ev_start, hipEventDisableTiming));
         SESSD_HIP_TRY(hipEventCreateWithFlags(&P->ev_vg, hipEventDisableTiming));
         P->ev_build.assign(P->stages.size(), nullptr);

@@ -112,7 +112,9 @@ class SubmConv3dLayerPlugin : public ConvPluginBase {
                       const void* const* inputs, void* const* outputs,
                       const void* rulebook_workspace, hipStream_t stream);
     // enqueue = enqueueBuild (coordinates -> rulebook) + enqueueGemm (features)
-    int enqueueBuild(const int32_t* coors, const int32_t* voxel_num, void* workspace, hipStream_t stream);
+    int enqueueBuild(const int32_t* coors, const int32_t* voxel_num, void* workspace, hipStream_t stream,
+                     bool prefilled = false);
+    void collectFill(void* workspace, FillArgs& f) const;
     int enqueueGemm(const void* in_feat, void* out_feat, const int32_t* voxel_num,
                     const void* rulebook_workspace, hipStream_t stream);
     int exportRulebook(const void* workspace, int32_t* indice_pairs, uint32_t* indice_num,
@@ -150,7 +152,8 @@ class SparseConv3dLayerPlugin : public ConvPluginBase {
                        hipStream_t stream) const;
     int countPairs(const void* workspace, uint32_t* indice_num, hipStream_t stream) const;
     int enqueueBuild(const int32_t* coors, const int32_t* voxel_num, int32_t* out_coors, int32_t* out_num,
-                     void* workspace, hipStream_t stream);
+                     void* workspace, hipStream_t stream, bool prefilled = false);
+    void collectFill(void* workspace, int32_t* out_coors, FillArgs& f) const;
     int enqueueGemm(const void* in_feat, void* out_feat, const int32_t* out_num, const void* workspace,
                     hipStream_t stream);
     size_t getSerializationSize() const;
@@ -181,7 +184,8 @@ class Sparse2DensePlugin {
                             const sessd_tensor_desc* outputs, int nbOutputs) const;
     int enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
                 const void* const* inputs, void* const* outputs, void* workspace,
-                hipStream_t stream);
+                hipStream_t stream, bool prefilled = false);
+    void collectFill(void* dense, void* workspace, FillArgs& f) const;
     size_t getSerializationSize() const;
     void serialize(void* buffer) const;
 

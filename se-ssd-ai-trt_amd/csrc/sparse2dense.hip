@@ -93,9 +93,15 @@ size_t Sparse2DensePlugin::getWorkspaceSize(const sessd_tensor_desc*, int, const
     return kWorkspaceAlign;
 }
 
+void Sparse2DensePlugin::collectFill(void* dense, void* workspace, FillArgs& f) const {
+    const uint64_t elems = (uint64_t)feature_map_channel_ * feature_map_size_z_ * feature_map_size_y_ * feature_map_size_x_;
+    f.add(dense, elems * dtype_size(out_type_) / 4, 0);  // sparse2Dense.cu:242
+    if (workspace) f.add(workspace, 4, 0);
+}
+
 int Sparse2DensePlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
                                 const void* const* inputs, void* const* outputs, void* workspace,
-                                hipStream_t stream) {
+                                hipStream_t stream, bool prefilled) {
     if (!inputDesc || !outputDesc || !inputs || !outputs || !inputs[0] || !inputs[1] || !inputs[2] || !outputs[0])
         return fail(SESSD_E_INVALID, "sparse2dense.enqueue: null argument");
     if (inputDesc[0].d[0] != 1) return fail(SESSD_E_UNSUPPORTED, "sparse2dense.enqueue: batch size must be 1");
@@ -112,10 +118,11 @@ int Sparse2DensePlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_
         return fail(SESSD_E_INVALID, "sparse2dense.enqueue: tensors must be 16-byte aligned");
     int32_t* status = static_cast<int32_t*>(workspace);
 
-    FillArgs f;
-    f.add(outputs[0], bytes / 4, 0);  // sparse2Dense.cu:242
-    if (status) f.add(status, 4, 0);
-    SESSD_TRY(launch_fill(f, stream));
+    if (!prefilled) {
+        FillArgs f;
+        collectFill(outputs[0], workspace, f);
+        SESSD_TRY(launch_fill(f, stream));
+    }
     const unsigned blocks = (unsigned)(((uint64_t)max_voxels * C + kBlock - 1) / kBlock);
     const int32_t* coors = static_cast<const int32_t*>(inputs[1]);
     const int32_t* num = static_cast<const int32_t*>(inputs[2]);

@@ -342,8 +342,16 @@ size_t SparseConv3dLayerPlugin::statusOffset() const { return carve(nullptr).met
 
 // The two halves of enqueue (see SubmConv3dLayerPlugin::enqueueBuild): output sites + rulebook from the
 // coordinates, then the GEMM over the features.
+void SparseConv3dLayerPlugin::collectFill(void* workspace, int32_t* out_coors, FillArgs& f) const {
+    const Layout L = carve(workspace);
+    f.add(L.keys, (uint64_t)L.cap * 2, kEmpty);
+    f.add(L.nbr, (uint64_t)kernel_volume_ * max_voxels_, kEmpty);  // -1 = no input at this offset
+    f.add(L.meta, 4, 0);
+    if (!(flags_ & SESSD_FLAG_SKIP_PAD_ROWS)) f.add(out_coors, (uint64_t)max_voxels_ * 4, 0);  // :668
+}
+
 int SparseConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* voxel_num, int32_t* out_coors,
-                                          int32_t* out_num, void* workspace, hipStream_t stream) {
+                                          int32_t* out_num, void* workspace, hipStream_t stream, bool prefilled) {
     if (!coors || !voxel_num || !out_coors || !out_num || !workspace)
         return fail(SESSD_E_INVALID, "sparseconv3d.build: null pointer");
     if (reinterpret_cast<uintptr_t>(out_coors) & 15)
@@ -359,12 +367,11 @@ int SparseConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* v
     P.max_voxels = max_voxels_;
     P.dilation = dilation_;
 
-    FillArgs f;
-    f.add(L.keys, (uint64_t)L.cap * 2, kEmpty);
-    f.add(L.nbr, (uint64_t)kernel_volume_ * max_voxels_, kEmpty);  // -1 = no input at this offset
-    f.add(L.meta, 4, 0);
-    if (!(flags_ & SESSD_FLAG_SKIP_PAD_ROWS)) f.add(out_coors, (uint64_t)max_voxels_ * 4, 0);  // :668
-    SESSD_TRY(launch_fill(f, stream));
+    if (!prefilled) {
+        FillArgs f;
+        collectFill(workspace, out_coors, f);
+        SESSD_TRY(launch_fill(f, stream));
+    }
     const dim3 grid(L.n_blocks), block(kBlock);
     hipLaunchKernelGGL(sp_insert, grid, block, 0, stream, coors, voxel_num, P, t, L.cand, L.meta);
     hipLaunchKernelGGL(sp_flags, grid, block, 0, stream, voxel_num, P, t, L.cand, L.first_words, L.block_counts);

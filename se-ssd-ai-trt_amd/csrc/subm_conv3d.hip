@@ -221,16 +221,25 @@ size_t SubmConv3dLayerPlugin::statusOffset() const { return carve(nullptr).meta_
 
 // The two halves of enqueue.  The rulebook depends only on the coordinates, the GEMM only on the
 // rulebook and the features: a pipeline may run the halves of different layers on different streams.
+// what enqueueBuild clears before it launches anything: a caller that batches the clears of many layers
+// into one launch collects them with this and passes prefilled = true
+void SubmConv3dLayerPlugin::collectFill(void* workspace, FillArgs& f) const {
+    const Layout L = carve(workspace);
+    f.add(L.keys, (uint64_t)L.cap * 2, kEmpty);
+    f.add(L.meta, 4, 0);
+}
+
 int SubmConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* voxel_num, void* workspace,
-                                        hipStream_t stream) {
+                                        hipStream_t stream, bool prefilled) {
     if (!coors || !voxel_num || !workspace) return fail(SESSD_E_INVALID, "submconv3d.build: null pointer");
     const Layout L = carve(workspace);
     const HashTable t = make_hash(L.keys, L.vals, L.cap);
     const Grid3 g{out_shape_x_, out_shape_y_, out_shape_z_};
-    FillArgs f;
-    f.add(L.keys, (uint64_t)L.cap * 2, kEmpty);
-    f.add(L.meta, 4, 0);
-    SESSD_TRY(launch_fill(f, stream));
+    if (!prefilled) {
+        FillArgs f;
+        collectFill(workspace, f);
+        SESSD_TRY(launch_fill(f, stream));
+    }
     const int row_blocks = ceil_div(max_voxels_, kBlock);
     hipLaunchKernelGGL(subm_insert, dim3(row_blocks), dim3(kBlock), 0, stream, coors, voxel_num, max_voxels_,
                        g, t, L.meta);
