@@ -285,6 +285,13 @@ size_t sessd_sparse2dense_workspace_size(const sessd_sparse2dense* h, const sess
 int sessd_sparse2dense_enqueue(sessd_sparse2dense* h, const sessd_tensor_desc* inDesc,
                                const sessd_tensor_desc* outDesc, const void* const* inputs,
                                void* const* outputs, void* workspace, sessd_stream_t stream);
+/* Folds the reference's ZeroPad2dPlugin (zeroPad2d.cu:183-244; creator field zero_padding_2d_size =
+ * top, bottom, left, right, zeroPad2d.cu:311, se-ssd-ai-trt.cpp:615-619), which the reference runs
+ * right after sparse2Dense (se-ssd-ai-trt.cpp:1253), into this plugin: the output becomes
+ * [1, C*D, H + top + bottom, W + left + right] with a zero border and the unpadded tensor is never
+ * written.  Call before configure.  All zeros (the default) = the reference's Sparse2DensePlugin. */
+int sessd_sparse2dense_set_padding(sessd_sparse2dense* h, int32_t top, int32_t bottom, int32_t left,
+                                   int32_t right);
 /* replaces destroy (sparse2Dense.cu:297-300) */
 void sessd_sparse2dense_destroy(sessd_sparse2dense* h);
 
@@ -326,6 +333,9 @@ typedef struct sessd_pipeline_desc {
                                     voxelizer's cap: strided layers can produce more sites than they get */
     int32_t overlap_streams;     /* run the coordinate chain (voxelizer + rulebook builds) on a second
                                     stream owned by the pipeline, overlapping the GEMMs of earlier layers */
+    int32_t dense_padding[4];    /* top, bottom, left, right: zero border around the dense tensor
+                                    (sessd_sparse2dense_set_padding); the reference network uses 1,1,1,1
+                                    (params.h:200-203).  The caller's dense buffer has the padded size */
 } sessd_pipeline_desc;
 
 /* Fills `layers[14]` with the reference backbone (params.h:39-192) and `dense`/`voxelgen` with
@@ -334,6 +344,40 @@ int sessd_reference_backbone(sessd_layer_spec* layers, int max_layers,
                              sessd_voxelgen_desc* voxelgen, sessd_sparse2dense_desc* dense);
 
 int sessd_pipeline_create(const sessd_pipeline_desc* desc, sessd_pipeline** out);
+
+/* ------------------------------------------------------------------------------------------ */
+/* `.wts` weight files and BatchNorm folding (host side; no GPU call)                          */
+/* ------------------------------------------------------------------------------------------ */
+/* replaces loadWeights (se-ssd-ai-trt.cpp:276-314; writer: tools/gen_wts.py:86-99): text, the blob
+ * count, then per blob `name count` and `count` tokens of big-endian hex float bits.  Malformed input
+ * is an error code where the reference asserts. */
+typedef struct sessd_wts sessd_wts;
+int sessd_wts_load(const char* path, sessd_wts** out);
+int sessd_wts_parse(const char* text, size_t length, sessd_wts** out);
+int sessd_wts_count(const sessd_wts* w);
+/* blob names in file order; the pointer lives as long as the handle */
+int sessd_wts_name(const sessd_wts* w, int index, const char** name);
+/* replaces weightMap[name] (e.g. se-ssd-ai-trt.cpp:1148); an unknown name is an error, not an empty blob */
+int sessd_wts_find(const sessd_wts* w, const char* name, const float** values, int64_t* count);
+void sessd_wts_destroy(sessd_wts* w);
+/* replaces the folding in add_batchNorm1d_relu (se-ssd-ai-trt.cpp:808-824), FP32 arithmetic:
+ * scale = gamma / sqrtf(var + eps), shift = beta - mean * gamma / sqrtf(var + eps) */
+int sessd_fold_batchnorm(const float* gamma, const float* beta, const float* mean, const float* var,
+                         int32_t n, float eps, float* scale, float* shift);
+/* replaces loadData + the point count of its caller (se-ssd-ai-trt.cpp:1515-1559, 1849-1850): reads a
+ * headerless float32 [n][point_features] file (KITTI velodyne `.bin`: x,y,z,intensity) into the host
+ * buffer points[max_points][point_features], zero-fills the rest, and returns n = bytes / (4 *
+ * point_features).  A file that does not fit is an error (the reference exits). */
+int sessd_load_frame(const char* path, float* points, int32_t max_points, int32_t point_features,
+                     int32_t* points_size);
+/* replaces the weightMap lookups of the reference's network builder (se-ssd-ai-trt.cpp:1147-1249):
+ * layer l takes `<prefix><conv_index[l]>.weight` and the BatchNorm blobs `<prefix><conv_index[l]+1>.
+ * {weight,bias,running_mean,running_var}`, folded with `eps` (the reference passes 1e-5) + ReLU.
+ * prefix NULL = "backbone.middle_conv."; conv_index NULL = 0,3,6,...,39 (needs n_layers == 14).
+ * desc->weights/scale/shift/relu are ignored. */
+int sessd_pipeline_create_from_wts(const sessd_pipeline_desc* desc, const sessd_wts* wts,
+                                   const char* prefix, const int32_t* conv_index, float eps,
+                                   sessd_pipeline** out);
 /* points f32[max_points,point_features], points_size i32[1], dense [C*D,H,W]: device pointers */
 int sessd_pipeline_enqueue(sessd_pipeline* h, const void* points, const void* points_size,
                            void* dense, sessd_stream_t stream);

@@ -27,6 +27,7 @@
 //   oracle_scale_shift_relu / fold_bn   closed form (the reference has no test at this boundary:
 //                                       TensorRT IScaleLayer semantics are the textbook ones)
 //   oracle_sparse2dense                 closed-form index + inverse gather
+//   oracle_zero_pad2d                   equality with torch.nn.functional.pad (constant 0)
 //   oracle_frame                        composition of the above (checked against calling them
 //                                       one by one)
 
@@ -353,13 +354,15 @@ void oracle_round_to_half(float* x, int64_t n) {
     for (int64_t i = 0; i < n; ++i) x[i] = round_to_half(x[i]);
 }
 
-// se-ssd-ai-trt.cpp:816-824 -- BatchNorm folding on the host: gamma/sqrt(var+eps) evaluated with
-// the double sqrt and stored as float.
+// se-ssd-ai-trt.cpp:816-824 -- BatchNorm folding on the host.  The file includes <cmath> and is
+// `using namespace std` (:24,29), so `sqrt(var[i] + eps)` on a float argument is the float overload
+// and both expressions are evaluated in FP32, left to right: gamma / sqrtf(var + eps) and
+// beta - (mean * gamma) / sqrtf(var + eps).  `eps` arrives as a float parameter (:808).
 void oracle_fold_bn(const float* gamma, const float* beta, const float* mean, const float* var,
                     float eps, int32_t c, float* scale, float* shift) {
     for (int i = 0; i < c; ++i) {
-        scale[i] = (float)(gamma[i] / sqrt((double)(var[i] + eps)));
-        shift[i] = (float)(beta[i] - mean[i] * gamma[i] / sqrt((double)(var[i] + eps)));
+        scale[i] = gamma[i] / sqrtf(var[i] + eps);
+        shift[i] = beta[i] - mean[i] * gamma[i] / sqrtf(var[i] + eps);
     }
 }
 
@@ -391,6 +394,22 @@ void oracle_sparse2dense(const float* feat, const int32_t* coors, int32_t n, int
             dense[(size_t)b * channels * W * H * D + ((size_t)(i * D) + z) * W * H + (size_t)y * W + x] =
                 feat[(size_t)v * channels + i];
         }
+    }
+}
+
+// zeroPad2d.cu:183-244 -- out[c][y + top][x + left] = in[c][y][x] over a zero-filled
+// [channels][height + top + bottom][width + left + right] tensor (the memset of :230, then one
+// thread per (y,x) looping over the channels, :188-200).
+void oracle_zero_pad2d(const float* in, int32_t channels, int32_t height, int32_t width, int32_t top,
+                       int32_t bottom, int32_t left, int32_t right, float* out) {
+    const int output_height = height + top + bottom, output_width = width + left + right;
+    std::memset(out, 0, sizeof(float) * (size_t)channels * output_height * output_width);
+    for (int idx = 0; idx < height * width; ++idx) {
+        const int height_index = idx / width, width_index = idx % width;
+        const int oh = height_index + top, ow = width_index + left;
+        for (int i = 0; i < channels; ++i)
+            out[(size_t)i * output_height * output_width + (size_t)oh * output_width + ow] =
+                in[(size_t)i * height * width + (size_t)height_index * width + width_index];
     }
 }
 

@@ -251,6 +251,10 @@ int sessd_sparse2dense_enqueue(sessd_sparse2dense* h, const sessd_tensor_desc* i
     NEED(h, "null handle");
     return H_S2D(h)->enqueue(inDesc, outDesc, inputs, outputs, workspace, static_cast<hipStream_t>(stream));
 }
+int sessd_sparse2dense_set_padding(sessd_sparse2dense* h, int32_t top, int32_t bottom, int32_t left, int32_t right) {
+    NEED(h, "null handle");
+    return H_S2D(h)->setPadding(top, bottom, left, right);
+}
 void sessd_sparse2dense_destroy(sessd_sparse2dense* h) { delete H_S2D(h); }
 
 }  // extern "C"

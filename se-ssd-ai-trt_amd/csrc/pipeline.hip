@@ -318,11 +318,12 @@ static int build_pipeline(const sessd_pipeline_desc& d, Pipeline* P) {
     Sparse2DensePlugin* s2d = nullptr;
     SESSD_TRY(Sparse2DensePlugin::create(d.dense, &s2d));
     P->s2d.reset(s2d);
+    SESSD_TRY(s2d->setPadding(d.dense_padding[0], d.dense_padding[1], d.dense_padding[2], d.dense_padding[3]));
     P->s2d_in[0] = make_desc({1, V, in_ch}, in_type);
     P->s2d_in[1] = make_desc({1, V, 4}, SESSD_INT32);
     P->s2d_in[2] = make_desc({1}, SESSD_INT32);
-    P->s2d_out[0] = make_desc({1, d.dense.feature_map_channel * d.dense.feature_map_size[2],
-                               d.dense.feature_map_size[1], d.dense.feature_map_size[0]}, ft);
+    P->s2d_out[0] = make_desc({1, d.dense.feature_map_channel * d.dense.feature_map_size[2], s2d->outHeight(),
+                               s2d->outWidth()}, ft);
     SESSD_TRY(s2d->configurePlugin(P->s2d_in, 3, P->s2d_out, 1));
     SESSD_TRY(P->s2d_ws.alloc(s2d->getWorkspaceSize(P->s2d_in, 3, P->s2d_out, 1)));
     total += P->s2d_ws.bytes;

@@ -189,8 +189,18 @@ class Sparse2DensePlugin {
     size_t getSerializationSize() const;
     void serialize(void* buffer) const;
 
+    int setPadding(int top, int bottom, int left, int right);
+    int outHeight() const { return feature_map_size_y_ + zero_padding_2d_top_ + zero_padding_2d_bottom_; }
+    int outWidth() const { return feature_map_size_x_ + zero_padding_2d_left_ + zero_padding_2d_right_; }
+    bool padded() const {
+        return (zero_padding_2d_top_ | zero_padding_2d_bottom_ | zero_padding_2d_left_ | zero_padding_2d_right_) != 0;
+    }
+
     int feature_map_size_x_ = 0, feature_map_size_y_ = 0, feature_map_size_z_ = 0;
     int feature_map_channel_ = 0;
+    // border written around every channel plane: the reference's ZeroPad2dPlugin (zeroPad2d.cu:183-244),
+    // which follows sparse2Dense in its network (se-ssd-ai-trt.cpp:1253), folded into this scatter
+    int zero_padding_2d_top_ = 0, zero_padding_2d_bottom_ = 0, zero_padding_2d_left_ = 0, zero_padding_2d_right_ = 0;
     int in_type_ = SESSD_FLOAT, out_type_ = SESSD_FLOAT;
 };
 

@@ -73,6 +73,20 @@ def lib():
     L.sessd_submconv3d_enqueue_shared.argtypes = [vp, TD, TD, VPP, VPP, vp, vp]
     L.sessd_sparseconv3d_create.argtypes = [C.POINTER(D.SparseConv3dDesc), vp, VPP]
     L.sessd_sparse2dense_create.argtypes = [C.POINTER(D.Sparse2DenseDesc), VPP]
+    L.sessd_sparse2dense_set_padding.argtypes = [C.c_void_p] + [C.c_int32] * 4
+    L.sessd_sparse2dense_set_padding.restype = C.c_int
+    FPP = C.POINTER(C.POINTER(C.c_float))
+    L.sessd_wts_load.argtypes = [C.c_char_p, VPP]
+    L.sessd_wts_parse.argtypes = [C.c_char_p, sz, VPP]
+    L.sessd_wts_count.argtypes = [vp]
+    L.sessd_wts_name.argtypes = [vp, C.c_int, C.POINTER(C.c_char_p)]
+    L.sessd_wts_find.argtypes = [vp, C.c_char_p, FPP, C.POINTER(C.c_int64)]
+    L.sessd_wts_destroy.argtypes = [vp]
+    L.sessd_wts_destroy.restype = None
+    FP1 = C.POINTER(C.c_float)
+    L.sessd_fold_batchnorm.argtypes = [FP1, FP1, FP1, FP1, i32, C.c_float, FP1, FP1]
+    L.sessd_pipeline_create_from_wts.argtypes = [C.POINTER(D.PipelineDesc), vp, C.c_char_p, C.POINTER(i32), C.c_float, VPP]
+    L.sessd_load_frame.argtypes = [C.c_char_p, FP1, i32, i32, C.POINTER(i32)]
     L.sessd_reference_backbone.argtypes = [C.POINTER(D.LayerSpec), C.c_int, C.POINTER(D.VoxelGenDesc),
                                            C.POINTER(D.Sparse2DenseDesc)]
     L.sessd_pipeline_create.argtypes = [C.POINTER(D.PipelineDesc), VPP]
@@ -308,17 +322,23 @@ class SparseConv3d(_Conv):
 class Sparse2Dense(_Plugin):
     kind = "sparse2dense"
 
-    def __init__(self, feature_map_size_xyz=B.DENSE_SIZE_XYZ, feature_map_channel=B.DENSE_CHANNEL):
+    def __init__(self, feature_map_size_xyz=B.DENSE_SIZE_XYZ, feature_map_channel=B.DENSE_CHANNEL,
+                 padding=(0, 0, 0, 0)):
         d = B.dense_desc(feature_map_size_xyz, feature_map_channel)
         h = C.c_void_p()
         check(lib().sessd_sparse2dense_create(C.byref(d), C.byref(h)))
         super().__init__(h)
         self.size, self.channel = tuple(feature_map_size_xyz), feature_map_channel
+        self.padding = tuple(int(v) for v in padding)  # top, bottom, left, right
+        if any(self.padding):
+            check(lib().sessd_sparse2dense_set_padding(self.h, *self.padding))
 
     def __call__(self, feat, coors, voxel_num, out_dtype=None, stream=None):
         torch = _torch()
         W, H, Dz = self.size
-        dense = torch.empty((self.channel * Dz, H, W), dtype=out_dtype or feat.dtype, device=feat.device)
+        top, bottom, left, right = self.padding
+        dense = torch.empty((self.channel * Dz, H + top + bottom, W + left + right),
+                            dtype=out_dtype or feat.dtype, device=feat.device)
         ins = [feat, coors, voxel_num]
         self.configure(ins, [dense])
         self.enqueue(ins, [dense], stream)
@@ -343,13 +363,67 @@ def make_conv(layer: B.Layer, weights, prev_grid_xyz, max_voxels, scale=None, sh
     return p
 
 
+class WeightFile:
+    """A parsed `.wts` file (the reference's text weight format, se-ssd-ai-trt.cpp:276-314)."""
+
+    def __init__(self, path=None, text=None):
+        self.h = C.c_void_p()
+        if path is not None:
+            check(lib().sessd_wts_load(os.fsencode(path), C.byref(self.h)))
+        else:
+            data = text.encode() if isinstance(text, str) else bytes(text)
+            check(lib().sessd_wts_parse(data, len(data), C.byref(self.h)))
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().sessd_wts_destroy(self.h)
+            self.h = None
+
+    def names(self):
+        out = []
+        for i in range(lib().sessd_wts_count(self.h)):
+            s = C.c_char_p()
+            check(lib().sessd_wts_name(self.h, i, C.byref(s)))
+            out.append(s.value.decode())
+        return out
+
+    def __getitem__(self, name):
+        p = C.POINTER(C.c_float)()
+        n = C.c_int64()
+        check(lib().sessd_wts_find(self.h, name.encode(), C.byref(p), C.byref(n)))
+        if n.value == 0:
+            return np.zeros(0, np.float32)
+        return np.ctypeslib.as_array(p, shape=(n.value,)).copy()
+
+
+def load_frame(path, max_points, point_features=4, out=None):
+    """One frame file -> (points float32[max_points, point_features] host array, number of points); see
+    sessd_load_frame.  `out` may be a pinned torch tensor's numpy view to read straight into it."""
+    pts = out if out is not None else np.empty((max_points, point_features), np.float32)
+    assert pts.dtype == np.float32 and pts.flags["C_CONTIGUOUS"] and pts.shape == (max_points, point_features)
+    n = C.c_int32()
+    check(lib().sessd_load_frame(os.fsencode(path), pts.ctypes.data_as(C.POINTER(C.c_float)), max_points,
+                                 point_features, C.byref(n)))
+    return pts, n.value
+
+
+def fold_batchnorm(gamma, beta, mean, var, eps=1e-5):
+    """The library's BatchNorm folding (se-ssd-ai-trt.cpp:808-824) -> (scale, shift)."""
+    g, b, m, v = (np.ascontiguousarray(a, np.float32) for a in (gamma, beta, mean, var))
+    sc, sh = np.empty_like(g), np.empty_like(g)
+    FP = C.POINTER(C.c_float)
+    check(lib().sessd_fold_batchnorm(*[a.ctypes.data_as(FP) for a in (g, b, m, v)], g.size, C.c_float(eps),
+                                     sc.ctypes.data_as(FP), sh.ctypes.data_as(FP)))
+    return sc, sh
+
+
 class Pipeline:
     """voxelGenerator -> conv stack -> sparse2Dense, owned and run by the library (C++)."""
 
     def __init__(self, layers, weights: B.Weights, max_points, max_voxels=B.MAX_VOXELS, point_features=4,
                  feature_dtype="fp32", relu=True, share_rulebooks=True, skip_pad_rows=False, use_graph=False,
                  dense_size_xyz=B.DENSE_SIZE_XYZ, max_pts_per_voxel=B.MAX_NUM_POINTS_PER_VOXEL,
-                 use_epilogue=True, overlap_streams=False, voxel_cap=None):
+                 use_epilogue=True, overlap_streams=False, voxel_cap=None, dense_padding=(0, 0, 0, 0)):
         """max_voxels = rows of every conv-layer tensor; voxel_cap (default: max_voxels) = the voxelizer's
         own limit."""
         torch = _torch()
@@ -359,9 +433,13 @@ class Pipeline:
         self.dtype = torch.float16 if feature_dtype in ("fp16", "half", torch.float16) else torch.float32
         n = len(self.layers)
         self._specs = B.layer_specs(self.layers)
-        self._w = [np.ascontiguousarray(w, np.float32) for w in weights.w]
-        self._s = [np.ascontiguousarray(s, np.float32) for s in weights.scale]
-        self._b = [np.ascontiguousarray(s, np.float32) for s in weights.shift]
+        from_file = isinstance(weights, WeightFile)
+        if from_file:
+            self._w = self._s = self._b = []
+        else:
+            self._w = [np.ascontiguousarray(w, np.float32) for w in weights.w]
+            self._s = [np.ascontiguousarray(s, np.float32) for s in weights.scale]
+            self._b = [np.ascontiguousarray(s, np.float32) for s in weights.shift]
         FP = C.POINTER(C.c_float)
         arr = lambda xs: (FP * max(n, 1))(*[x.ctypes.data_as(FP) for x in xs])  # noqa: E731
         d = D.PipelineDesc()
@@ -369,10 +447,11 @@ class Pipeline:
         d.layer_max_voxels = max_voxels
         d.max_points, d.point_features, d.n_layers = max_points, point_features, n
         d.layers = self._specs
-        d.weights = arr(self._w)
-        if use_epilogue:
-            d.scale = arr(self._s)
-            d.shift = arr(self._b)
+        if not from_file:
+            d.weights = arr(self._w)
+            if use_epilogue:
+                d.scale = arr(self._s)
+                d.shift = arr(self._b)
         d.relu = int(relu)
         d.feature_dtype = D.SESSD_HALF if self.dtype == torch.float16 else D.SESSD_FLOAT
         c_last = self.layers[-1].cout if n else 4
@@ -381,9 +460,17 @@ class Pipeline:
         d.flags = D.SESSD_FLAG_SKIP_PAD_ROWS if skip_pad_rows else 0
         d.use_graph = int(use_graph)
         d.overlap_streams = int(overlap_streams)
-        self.dense_shape = (c_last * dense_size_xyz[2], dense_size_xyz[1], dense_size_xyz[0])
+        top, bottom, left, right = (int(v) for v in dense_padding)
+        d.dense_padding = (C.c_int32 * 4)(top, bottom, left, right)
+        self.dense_shape = (c_last * dense_size_xyz[2], dense_size_xyz[1] + top + bottom,
+                            dense_size_xyz[0] + left + right)
         self.h = C.c_void_p()
-        check(lib().sessd_pipeline_create(C.byref(d), C.byref(self.h)))
+        if from_file:  # conv weights and BatchNorm statistics by the reference's blob names, folded by the library
+            idx = (C.c_int32 * n)(*[B.conv_index(l) for l in self.layers])
+            check(lib().sessd_pipeline_create_from_wts(C.byref(d), weights.h, None, idx, C.c_float(1e-5),
+                                                       C.byref(self.h)))
+        else:
+            check(lib().sessd_pipeline_create(C.byref(d), C.byref(self.h)))
 
     def new_dense(self, device="cuda"):
         torch = _torch()
@@ -398,6 +485,13 @@ class Pipeline:
         ch = C.c_int32()
         check(lib().sessd_pipeline_layer_io(self.h, layer, C.byref(f), C.byref(c), C.byref(n), C.byref(w), C.byref(ch)))
         return f.value, c.value, n.value, w.value, ch.value
+
+    def layer_count(self, layer):
+        """Active rows a layer produced in the last enqueue (layer = -1: the voxelizer)."""
+        _torch().cuda.synchronize()
+        num = np.zeros(1, np.int32)
+        _hip_d2h(num, self.layer_io(layer)[2])
+        return int(num[0])
 
     def read_layer(self, layer):
         """Copy a layer's output of the last enqueue to the host: feat[n,C] float32, coors[n,4], n."""

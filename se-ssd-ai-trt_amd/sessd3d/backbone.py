@@ -64,6 +64,12 @@ def reference_layers(width_mult: int = 1, subm_per_64_stage: int = 3) -> List[La
     return L
 
 
+def conv_index(layer: Layer) -> int:
+    """Index of the layer inside the reference's `backbone.middle_conv` Sequential (its name's number:
+    se-ssd-ai-trt.cpp:1147-1249); the layer's BatchNorm is index + 1."""
+    return int("".join(ch for ch in layer.name if ch.isdigit()))
+
+
 def conv_out_size(n, k, s, p):
     """spconv's output extent for one axis: (n + 2p - k)//s + 1."""
     return (n + 2 * p - k) // s + 1
@@ -77,13 +83,13 @@ class Weights:
 
 
 def fold_bn(gamma, beta, mean, var, eps=1e-5):
-    """se-ssd-ai-trt.cpp:816-824: scale = gamma/sqrt(var+eps), shift = beta - mean*scale, the sqrt
-    in double precision, the results stored as float32."""
+    """se-ssd-ai-trt.cpp:816-824: scale = gamma/sqrt(var+eps), shift = beta - mean*gamma/sqrt(var+eps),
+    every operation in float32 (the reference's `sqrt` on a float resolves to the float overload)."""
     gamma, beta, mean, var = (np.asarray(a, np.float32) for a in (gamma, beta, mean, var))
-    ve = (var + np.float32(eps)).astype(np.float64)
-    scale = (gamma.astype(np.float64) / np.sqrt(ve)).astype(np.float32)
-    shift = (beta.astype(np.float64) - mean.astype(np.float64) * gamma.astype(np.float64) / np.sqrt(ve)).astype(np.float32)
-    return scale, shift
+    root = np.sqrt(var + np.float32(eps), dtype=np.float32)
+    scale = gamma / root
+    shift = beta - (mean * gamma) / root
+    return scale.astype(np.float32), shift.astype(np.float32)
 
 
 def random_weights(layers: List[Layer], seed: int = 0, w_std: float = 0.1, bn: bool = True) -> Weights:
@@ -140,3 +146,51 @@ def dense_desc(size_xyz=DENSE_SIZE_XYZ, channel=DENSE_CHANNEL):
         d.feature_map_size[i] = size_xyz[i]
     d.feature_map_channel = channel
     return d
+
+
+WTS_PREFIX = "backbone.middle_conv."
+
+
+def write_wts(path, blobs) -> None:
+    """Writes `{name: array}` in the reference's text weight format (tools/gen_wts.py:86-99): the blob
+    count, then per blob `name count` and the big-endian hex of every float32."""
+    with open(path, "w") as f:
+        f.write("%d\n" % len(blobs))
+        for name, v in blobs.items():
+            a = np.ascontiguousarray(v, np.float32).reshape(-1)
+            f.write("%s %d " % (name, a.size))
+            for word in a.view(np.uint32):
+                f.write(" %08x" % int(word))
+            f.write("\n")
+
+
+def random_state_dict(layers: List[Layer], seed: int = 0, w_std: float = 0.1):
+    """Seeded stand-in for the `backbone.middle_conv.*` entries of an SE-SSD checkpoint: conv weights
+    [kz,ky,kx,Cin,Cout] and BatchNorm1d weight/bias/running_mean/running_var (+ num_batches_tracked, which
+    the reference's generator also writes and its loader ignores)."""
+    rng = np.random.default_rng(seed)
+    sd = {}
+    for l in layers:
+        i = conv_index(l)
+        sd["%s%d.weight" % (WTS_PREFIX, i)] = (rng.standard_normal(l.ksize + (l.cin, l.cout)) * w_std).astype(np.float32)
+        sd["%s%d.weight" % (WTS_PREFIX, i + 1)] = rng.uniform(0.5, 1.5, l.cout).astype(np.float32)
+        sd["%s%d.bias" % (WTS_PREFIX, i + 1)] = rng.uniform(-0.1, 0.3, l.cout).astype(np.float32)
+        sd["%s%d.running_mean" % (WTS_PREFIX, i + 1)] = rng.uniform(-0.2, 0.2, l.cout).astype(np.float32)
+        sd["%s%d.running_var" % (WTS_PREFIX, i + 1)] = rng.uniform(0.5, 1.5, l.cout).astype(np.float32)
+        sd["%s%d.num_batches_tracked" % (WTS_PREFIX, i + 1)] = np.array([1234.0], np.float32)
+    return sd
+
+
+def weights_from_blobs(layers: List[Layer], get, eps: float = 1e-5) -> Weights:
+    """`get(name) -> flat float32 array` (a parsed weight file or a dict) -> per-layer [K,Cin,Cout] weights
+    and folded BatchNorm scale/shift, by the blob names the reference uses (se-ssd-ai-trt.cpp:1147-1249)."""
+    out = Weights()
+    for l in layers:
+        i = conv_index(l)
+        out.w.append(np.asarray(get("%s%d.weight" % (WTS_PREFIX, i)), np.float32).reshape(l.kvol, l.cin, l.cout))
+        bn = "%s%d" % (WTS_PREFIX, i + 1)
+        s, b = fold_bn(*(np.asarray(get(bn + k), np.float32).reshape(-1)
+                         for k in (".weight", ".bias", ".running_mean", ".running_var")), eps=eps)
+        out.scale.append(s)
+        out.shift.append(b)
+    return out

@@ -78,4 +78,5 @@ class PipelineDesc(C.Structure):
                 ("layers", C.POINTER(LayerSpec)), ("weights", FloatPP), ("scale", FloatPP),
                 ("shift", FloatPP), ("relu", C.c_int32), ("feature_dtype", C.c_int32),
                 ("dense", Sparse2DenseDesc), ("share_rulebooks", C.c_int32), ("flags", C.c_int32),
-                ("use_graph", C.c_int32), ("layer_max_voxels", C.c_int32), ("overlap_streams", C.c_int32)]
+                ("use_graph", C.c_int32), ("layer_max_voxels", C.c_int32), ("overlap_streams", C.c_int32),
+                ("dense_padding", C.c_int32 * 4)]

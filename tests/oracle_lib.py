@@ -155,6 +155,16 @@ def sparse2dense(feat, coors, n, size_xyz):
     return dense
 
 
+
+def zero_pad2d(x, top, bottom, left, right):
+    """x f32[channels, height, width] -> zero-bordered copy (the reference's ZeroPad2dPlugin)."""
+    a = np.ascontiguousarray(x, np.float32)
+    c, h, w = a.shape
+    out = np.empty((c, h + top + bottom, w + left + right), np.float32)
+    lib.oracle_zero_pad2d(_p(a, _f), C.c_int32(c), C.c_int32(h), C.c_int32(w), C.c_int32(top), C.c_int32(bottom),
+                          C.c_int32(left), C.c_int32(right), _p(out, _f))
+    return out
+
 def conv_layer(feat, coors, n, layer, w, scale, shift, max_voxels, relu=True):
     """One backbone layer through the oracle: rulebook, gather-GEMM-scatter, epilogue.
     -> out_feat[max_voxels,Cout], out_coors, out_n, pairs, num"""

@@ -376,6 +376,36 @@ def test_sparse_generic_stride1_and_corner_truncation():
         assert_features_close(out, O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), RTOL_FP32, str((k, s, p)))
 
 
+def test_sparse2dense_with_folded_zero_pad():
+    # sparse2Dense followed by ZeroPad2dPlugin (se-ssd-ai-trt.cpp:1253) in one scatter; a copy: bit-exact
+    rng = np.random.default_rng(12)
+    n, mv, c = 2739, 8192, 64
+    coors = F.random_active_voxels(n, (2, 200, 176), 9)
+    coors[:4] = [(0, 0, 0, 0), (0, 1, 199, 175), (0, 0, 199, 0), (0, 1, 0, 175)]      # the four corners
+    coors = np.unique(coors, axis=0)
+    n = len(coors)
+    feat = rng.uniform(0.1, 1, (n, c)).astype(np.float32)
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = np.zeros((mv, c), np.float32)
+    fbuf[:n] = feat
+    for pad in [(1, 1, 1, 1), (2, 0, 1, 3)]:
+        for dt in (torch.float32, torch.float16):
+            s2d = api.Sparse2Dense(padding=pad)
+            f = dev(fbuf).to(dt)
+            dense = s2d(f, dev(cbuf), dev(np.array([n], np.int32)))
+            torch.cuda.synchronize()
+            want = O.zero_pad2d(O.sparse2dense(to_np(f[:n].float()), coors, n, B.DENSE_SIZE_XYZ), *pad)
+            assert tuple(dense.shape) == want.shape
+            assert np.array_equal(to_np(dense.float()), want), (pad, dt)
+            assert s2d.status() == 0
+    # the output descriptor must carry the padded shape
+    s2d = api.Sparse2Dense(padding=(1, 1, 1, 1))
+    bad = torch.empty((128, 200, 176), dtype=torch.float32, device="cuda")
+    with pytest.raises(api.SessdError):
+        s2d.configure([dev(fbuf), dev(cbuf), dev(np.array([n], np.int32))], [bad])
+
+
 def test_sparse2dense():
     rng = np.random.default_rng(2)
     n, mv, c = 2739, 60000, 64

@@ -63,6 +63,31 @@ def test_full_backbone_small_frame(share, skip_pad):
     compare_with_oracle(pipe, dense, pts, layers, W, 16384, RTOL_FP32)
 
 
+@pytest.mark.parametrize("overlap", [False, True])
+def test_pipeline_writes_the_zero_padded_dense_tensor(overlap):
+    """dense_padding = the reference's ZeroPad2dPlugin (params.h:200-203: 1,1,1,1) folded into the last scatter:
+    the padded tensor must equal the oracle's sparse2dense -> zero_pad2d of the same rows, and its interior
+    the unpadded pipeline's output, bit for bit."""
+    pts = F.lidar_frame(4000, 21)
+    layers = B.reference_layers()
+    W = B.random_weights(layers, seed=6, w_std=0.05)
+    kw = dict(share_rulebooks=True, skip_pad_rows=True, overlap_streams=overlap, use_graph=overlap)
+    plain, dense, _ = run_pipeline(pts, layers, W, 4096, 16384, **kw)
+    pad = (1, 1, 1, 1)
+    pipe, padded, (p, n, stream) = run_pipeline(pts, layers, W, 4096, 16384, dense_padding=pad, **kw)
+    assert tuple(padded.shape) == (128, 202, 178)
+    feat, coors, m = pipe.read_layer(len(layers) - 1)
+    want = O.zero_pad2d(O.sparse2dense(feat, coors, m, B.DENSE_SIZE_XYZ), *pad)
+    assert np.array_equal(to_np(padded), want)
+    assert np.array_equal(to_np(padded)[:, 1:-1, 1:-1], to_np(dense))
+    # a second enqueue into a dirty buffer restores the zero border
+    padded.fill_(7.0)
+    with torch.cuda.stream(stream):
+        pipe.enqueue(p, n, padded, stream)
+    stream.synchronize()
+    assert np.array_equal(to_np(padded), want)
+
+
 def test_full_backbone_config3_frame_and_graph_replay():
     """BASELINE config 3: the 20 000-point frame (~17 k voxels) through the reference's 14 conv layers.
     The eager enqueue and repeated replays of the captured graph must give identical bits."""

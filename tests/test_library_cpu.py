@@ -94,6 +94,12 @@ def test_sparse2dense_host_side():
     d = B.dense_desc((176, 0, 2), 64)
     h = C.c_void_p()
     assert L.sessd_sparse2dense_create(C.byref(d), C.byref(h)) == D.SESSD_E_INVALID
+    # with a border the blob grows by a tagged trailer in the order of zeroPad2d.cu:283-290
+    p = api.Sparse2Dense(padding=(1, 2, 3, 4))
+    blob = p.serialize()
+    assert struct.unpack("<4i", blob[:16]) == (176, 200, 2, 64) and struct.unpack("<4i", blob[20:]) == (1, 2, 3, 4)
+    assert api.Sparse2Dense.deserialize(blob).serialize() == blob
+    assert L.sessd_sparse2dense_set_padding(p.h, -1, 0, 0, 0) == D.SESSD_E_INVALID
 
 
 def test_conv_create_validates_before_touching_the_gpu():

@@ -254,6 +254,19 @@ def test_sparse2dense_closed_form():
     assert dense[5 * 2 + coors[v, 1], coors[v, 2], coors[v, 3]] == feat[v, 5]
 
 
+def test_zero_pad2d_equals_torch_pad():
+    # zeroPad2d.cu:183-244 against the library routine, incl. asymmetric borders and the reference's 1,1,1,1
+    import torch
+    rng = np.random.default_rng(4)
+    for (c, h, w), (t, b, l, r) in [((128, 200, 176), (1, 1, 1, 1)), ((3, 5, 7), (2, 0, 1, 3)), ((1, 1, 1), (0, 0, 0, 0)),
+                                    ((4, 6, 2), (0, 3, 2, 0))]:
+        x = rng.uniform(0.5, 1.5, (c, h, w)).astype(np.float32)
+        want = torch.nn.functional.pad(torch.from_numpy(x), (l, r, t, b), mode="constant", value=0.0).numpy()
+        got = O.zero_pad2d(x, t, b, l, r)
+        assert got.shape == (c, h + t + b, w + l + r)
+        assert np.array_equal(got, want)
+
+
 def test_round_to_half_matches_numpy():
     rng = np.random.default_rng(0)
     x = np.concatenate([rng.normal(0, 1, 5000), rng.normal(0, 1e-5, 2000), rng.normal(0, 3e4, 2000),
