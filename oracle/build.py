@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 OUT = os.path.join(HERE, "_build", "libsessd_oracle.so")
 SRC = os.path.join(HERE, "sessd_oracle.cpp")
 # IEEE division, no FMA contraction: voxel coordinates and the summation order depend on it.
-FLAGS = ["-O2", "-fno-fast-math", "-ffp-contract=off", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra"]
+FLAGS = ["-O2", "-fno-fast-math", "-ffp-contract=off", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-fopenmp"]
 
 
 def build(force=True):

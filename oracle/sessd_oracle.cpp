@@ -63,6 +63,7 @@ struct DenseGrid {
     }
 };
 thread_local DenseGrid g_grid;
+int g_threads = 1;  // see oracle_set_threads
 
 // Round an FP32 value to the nearest IEEE binary16 value (ties to even, subnormals kept,
 // overflow to infinity) and return it as FP32.
@@ -326,18 +327,26 @@ int oracle_sparse_rulebook(const int32_t* coors, int32_t n, const int32_t* out_s
 // for k = 0..K-1 in order (:632-638).  out is zeroed over all max_voxels rows first (:594).
 // Per pair: s[c] = sum_j in[i][j]*W[k][j][c] with j ascending from 0.0f, then out[o][c] += s[c].
 // (The j loop is hoisted outside the c loop; each s[c] still accumulates in the same order.)
+//
+// Threads (oracle_set_threads, default 1): the pairs of ONE offset are split over threads.  Inside an
+// offset every output row occurs at most once (in = out*stride - pad + k is injective for fixed k), so
+// threads never share an output row and every out[o][c] still receives its terms in offset order: the
+// result is bit-identical for any thread count.  Used only to time a multi-core CPU baseline.
 void oracle_gather_gemm_scatter(const float* in_feat, const float* weights,
                                 const int32_t* indice_pairs, const uint32_t* indice_num, int32_t K,
                                 int32_t max_voxels, int32_t cin, int32_t cout, float* out_feat) {
+    if (cout > 512) std::abort();  // the per-pair accumulator below is a fixed array
     std::memset(out_feat, 0, sizeof(float) * (size_t)max_voxels * cout);
-    std::vector<float> s((size_t)cout);
     for (int k = 0; k < K; ++k) {
         const float* W = weights + (size_t)k * cin * cout;
         const int32_t* in_idx = indice_pairs + (size_t)k * 2 * max_voxels;
         const int32_t* out_idx = in_idx + max_voxels;
-        for (uint32_t a = 0; a < indice_num[k]; ++a) {
+        const int64_t pairs = indice_num[k];
+#pragma omp parallel for schedule(static) num_threads(g_threads) if (g_threads > 1 && pairs > 256)
+        for (int64_t a = 0; a < pairs; ++a) {
             const float* x = in_feat + (size_t)in_idx[a] * cin;
             float* y = out_feat + (size_t)out_idx[a] * cout;
+            float s[512];
             for (int c = 0; c < cout; ++c) s[c] = 0.0f;
             for (int j = 0; j < cin; ++j) {
                 const float xj = x[j];
@@ -348,6 +357,9 @@ void oracle_gather_gemm_scatter(const float* in_feat, const float* weights,
         }
     }
 }
+
+// Threads oracle_gather_gemm_scatter may use (>= 1); everything else stays sequential.
+void oracle_set_threads(int32_t n) { g_threads = n < 1 ? 1 : n; }
 
 // Test helper: nearest binary16 value of every element (ties to even), as FP32.
 void oracle_round_to_half(float* x, int64_t n) {

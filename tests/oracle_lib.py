@@ -156,6 +156,11 @@ def sparse2dense(feat, coors, n, size_xyz):
 
 
 
+def set_threads(n):
+    """Threads the gather-GEMM of the oracle may use (results do not depend on it)."""
+    lib.oracle_set_threads(C.c_int32(n))
+
+
 def zero_pad2d(x, top, bottom, left, right):
     """x f32[channels, height, width] -> zero-bordered copy (the reference's ZeroPad2dPlugin)."""
     a = np.ascontiguousarray(x, np.float32)

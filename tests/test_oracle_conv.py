@@ -254,6 +254,25 @@ def test_sparse2dense_closed_form():
     assert dense[5 * 2 + coors[v, 1], coors[v, 2], coors[v, 3]] == feat[v, 5]
 
 
+def test_gather_gemm_is_bit_identical_for_any_thread_count():
+    layer = B.reference_layers()[3]                      # subm9, 32 -> 32
+    rng = np.random.default_rng(6)
+    n, mv = 3000, 4096
+    coors = F.clustered_active_voxels(n, layer.out_shape[::-1], 5)
+    n = len(coors)
+    feat = rng.normal(size=(n, 32)).astype(np.float32)
+    w = rng.normal(0, 0.1, (27, 32, 32)).astype(np.float32)
+    pairs, num, _ = O.subm_rulebook(coors, n, layer.out_shape, mv)
+    assert int(num.sum()) > 3 * n
+    one = O.gather_gemm_scatter(feat, w, pairs, num, mv)
+    try:
+        O.set_threads(4)
+        four = O.gather_gemm_scatter(feat, w, pairs, num, mv)
+    finally:
+        O.set_threads(1)
+    assert np.array_equal(one.view(np.uint32), four.view(np.uint32))
+
+
 def test_zero_pad2d_equals_torch_pad():
     # zeroPad2d.cu:183-244 against the library routine, incl. asymmetric borders and the reference's 1,1,1,1
     import torch
