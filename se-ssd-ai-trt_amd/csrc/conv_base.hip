@@ -95,8 +95,8 @@ int ConvPluginBase::preparePacked() {
     return SESSD_OK;
 }
 
-int ConvPluginBase::runGemm(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* num_out,
-                            hipStream_t stream) {
+int ConvPluginBase::runGemm(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* tiles,
+                            const int32_t* num_out, hipStream_t stream) {
     GemmArgs a;
     a.in_feat = in_feat;
     a.out_feat = out_feat;
@@ -116,6 +116,7 @@ int ConvPluginBase::runGemm(const void* in_feat, void* out_feat, const int32_t* 
     a.relu = epi_.relu;
     a.write_pad_rows = (flags_ & SESSD_FLAG_SKIP_PAD_ROWS) ? 0 : 1;
     a.force_valu = (flags_ & SESSD_FLAG_FORCE_VALU) ? 1 : 0;
+    a.tiles = tiles;
     if (ev_gemm_begin_) SESSD_HIP_TRY(hipEventRecord(ev_gemm_begin_, stream));
     SESSD_TRY(launch_gather_gemm(a, stream));
     if (ev_gemm_end_) SESSD_HIP_TRY(hipEventRecord(ev_gemm_end_, stream));

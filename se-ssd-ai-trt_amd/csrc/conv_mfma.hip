@@ -2,9 +2,10 @@
 //
 //     out[o][:] = epilogue( sum_k  in[nbr[k][o]][:] @ W[k] )
 //
-// One workgroup (4 wave64) owns a tile of output rows and all Cout columns.  The tile height is chosen
-// per launch from the device-side row count so that every CU gets the same number of tiles
-// (tile_height()).
+// One workgroup (4 wave64) owns a tile of consecutive output rows and all Cout columns.  The number of
+// tiles is chosen per launch from the device-side row count so that every CU gets the same number of
+// tiles (tile_plan()); where the rulebook carries equal-work cuts (tile_cut.hip) the tiles follow them,
+// otherwise all tiles have the same length.
 //   * The tile's neighbour lists nbr[k][row0 .. row0+rows) are staged in LDS and compacted per offset
 //     with wave64 ballot + popcount: pair list k = the (input row, local output row) pairs of the rows
 //     that really have a neighbour at offset k.  Only those rows enter an MFMA block, so the matrix
@@ -42,26 +43,12 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 #ifndef SESSD_MFMA_TM
 #define SESSD_MFMA_TM 48
 #endif
-#ifndef SESSD_MFMA_TARGET
-#define SESSD_MFMA_TARGET 40
-#endif
 constexpr int kWaves = SESSD_MFMA_WAVES;
 constexpr int kTileRows = SESSD_MFMA_TM;        // capacity: most output rows a workgroup can own (<= 64)
-constexpr int kTargetRows = SESSD_MFMA_TARGET;  // tile height aimed for when choosing tiles per CU
 constexpr int kMaxBlk = (kTileRows + 15) / 16;  // MFMA row blocks an offset can need
 constexpr int kMaxK = 27;
 
-// Tile height for `n` active rows on `num_cu` compute units: the rows are split into num_cu * r tiles
-// of equal height, r = the smallest tiles-per-CU count that keeps the height at or below the target.
-// Every CU then gets the same number of tiles (a fixed 32-row tiling leaves e.g. 529 tiles for 256 CUs:
-// some CUs run three tiles, most two, and the kernel lasts as long as the three).
-static_assert(kTargetRows <= kTileRows && kTileRows <= 64, "tile height must fit the capacity and one wave");
-__host__ __device__ inline int tile_height(int n, int num_cu) {
-    if (n <= 0) return kTileRows;
-    const int r = (n + num_cu * kTargetRows - 1) / (num_cu * kTargetRows);
-    int h = (n + num_cu * r - 1) / (num_cu * r);
-    return h > kTileRows ? kTileRows : (h < 1 ? 1 : h);
-}
+static_assert(kGemmTargetRows <= kTileRows && kTileRows <= 64, "tile height must fit the capacity and one wave");
 
 // Per-dtype shape of one K-chunk: how many channels it spans, what a lane holds of it, and the MFMA
 // sequence that consumes it (w = weights fragment -> A operand, x = gathered-row fragment -> B operand).
@@ -122,7 +109,7 @@ __global__ void __launch_bounds__(kWaves * 64)
 conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict__ Wp,
           const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
           const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad,
-          int num_cu) {
+          int num_cu, const int32_t* __restrict__ tiles) {
     using C = Chunk<T, CIN>;
     using Vec = typename C::Vec;
     constexpr int G = CIN / C::kChannels;  // K-chunks of the inner dimension
@@ -160,10 +147,23 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
                 store4(out + (size_t)row * COUT + c4, o);
             }
     }
-    const int R = tile_height(n, num_cu);  // rows of this launch's tiles
-    const int row0 = blockIdx.x * R;
-    if (row0 >= n) return;
-    const int rows = n - row0 < R ? n - row0 : R;
+    // this workgroup's run of rows: from the rulebook's equal-work cuts, or equal lengths
+    int run_begin, run_end;
+    if (tiles && tiles[0] > 0) {
+        if ((int)blockIdx.x >= tiles[0]) return;
+        run_begin = tiles[4 + blockIdx.x];
+        run_end = tiles[5 + blockIdx.x];
+    } else {
+        const int R = tile_plan(n, num_cu).height;
+        run_begin = blockIdx.x * R;
+        run_end = run_begin + R < n ? run_begin + R : n;
+    }
+    const int i = lane & 15;  // pair inside a 16-pair block
+    const int q = lane >> 4;  // channel group inside a K-chunk
+    const Vec* wp = reinterpret_cast<const Vec*>(Wp) + lane;
+    // a run longer than the tile capacity (sparse stretches under equal-work cuts) is walked in pieces
+    for (int row0 = run_begin; row0 < run_end; row0 += kTileRows) {
+    const int rows = run_end - row0 < kTileRows ? run_end - row0 : kTileRows;
 
     // ---- stage + compact: a wave turns one offset's neighbour list into a pair list per step ----
     for (int k = wave; k < K; k += kWaves) {
@@ -181,9 +181,6 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
     for (int t = lane; t < rows * LDP / 4; t += 64) reinterpret_cast<float4*>(part)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
 
-    const int i = lane & 15;  // pair inside a 16-pair block
-    const int q = lane >> 4;  // channel group inside a K-chunk
-
     // offsets this wave handles: the non-empty ones, dealt round-robin (all wave-uniform)
     uint32_t my_mask = 0;
     {
@@ -195,7 +192,6 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
             }
     }
 
-    const Vec* wp = reinterpret_cast<const Vec*>(Wp) + lane;
     // gathered rows of all blocks of offset k -> operand registers (zeros for the padding pairs)
     auto load_a = [&](int k, int cnt, Vec (&a)[kMaxBlk][G]) {
 #pragma unroll
@@ -295,6 +291,8 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
         }
         store4(out + (size_t)(row0 + r) * COUT + c4, o);
     }
+    __syncthreads();  // the next piece reuses the lists and partial tiles
+    }
 }
 
 int compute_units() {
@@ -313,12 +311,11 @@ int compute_units() {
 template <typename T, int CIN, int COUT>
 int launch(const GemmArgs& a, hipStream_t stream) {
     const int num_cu = compute_units();
-    // tile_height() never cuts n <= max_voxels rows into more than num_cu * r_max tiles
-    const int r_max = ceil_div(a.max_voxels, (int64_t)num_cu * kTargetRows);
-    const unsigned blocks = (unsigned)(num_cu * (r_max < 1 ? 1 : r_max));
+    // tile_plan() never cuts n <= max_voxels rows into more tiles than it does max_voxels rows
+    const unsigned blocks = (unsigned)tile_plan(a.max_voxels, num_cu).count;
     hipLaunchKernelGGL((conv_mfma<T, CIN, COUT>), dim3(blocks), dim3(kWaves * 64), 0, stream,
                        static_cast<const T*>(a.in_feat), static_cast<T*>(a.out_feat), a.w_packed, a.nbr,
-                       a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows, num_cu);
+                       a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows, num_cu, a.tiles);
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;
 }
@@ -346,6 +343,8 @@ void chunk_shape(int dtype, int cin, int* channels, int* lane_elems) {
 }
 
 }  // namespace
+
+int gemm_compute_units() { return compute_units(); }
 
 size_t packed_weight_bytes(int K, int cin, int cout, int dtype) {
     if (!mfma_shape(K, cin, cout)) return 0;

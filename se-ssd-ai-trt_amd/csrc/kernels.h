@@ -21,7 +21,37 @@ struct GemmArgs {
     int relu;
     int write_pad_rows;      // rows >= *num_out get epilogue(0) (the reference zero-fills them)
     int force_valu;          // skip the MFMA kernels (cross-check)
+    const int32_t* tiles;    // tile cuts of this rulebook (launch_tile_cuts) or null: tiles of equal length
 };
+
+// Tiling of the MFMA gather-GEMM: n active rows on num_cu compute units are cut into num_cu * r tiles,
+// r = the smallest tiles-per-CU count that keeps the mean tile at or below the target height, so that every
+// CU gets the same number of tiles (a fixed 32-row tiling leaves e.g. 529 tiles for 256 CUs: some CUs run
+// three tiles, most two, and the kernel lasts as long as the three).
+constexpr int kGemmTargetRows = 40;
+struct TilePlan {
+    int count;   // tiles
+    int height;  // rows per tile when all tiles have the same length
+};
+__host__ __device__ inline TilePlan tile_plan(int n, int num_cu) {
+    TilePlan p;
+    if (n <= 0) {
+        p.count = num_cu;
+        p.height = 1;
+        return p;
+    }
+    const int r = (n + num_cu * kGemmTargetRows - 1) / (num_cu * kGemmTargetRows);
+    p.count = num_cu * r;
+    p.height = (n + p.count - 1) / p.count;
+    return p;
+}
+int gemm_compute_units();
+
+// equal-work tile cuts for the MFMA kernel, written into `region` (tile_cut_bytes() bytes of the layer's
+// workspace; its first word must be zero before the launch and stays zero when there are no active rows)
+size_t tile_cut_bytes(int max_voxels);
+int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, void* region,
+                     hipStream_t stream);
 
 // picks the kernel for the layer shape; returns SESSD_E_UNSUPPORTED for dtype pairs not covered
 int launch_gather_gemm(const GemmArgs& a, hipStream_t stream);

@@ -109,7 +109,7 @@ struct Pipeline {
             };
             for (auto& st : stages) {
                 if (!st->ws.p) continue;
-                if (f.n + 4 > FillArgs::kMaxRegions) SESSD_TRY(flush());
+                if (f.n + 5 > FillArgs::kMaxRegions) SESSD_TRY(flush());
                 if (st->subm) st->subm->collectFill(st->ws.p, f);
                 else st->sparse->collectFill(st->ws.p, static_cast<int32_t*>(st->coors.p), f);
             }

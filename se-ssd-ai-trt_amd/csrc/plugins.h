@@ -57,6 +57,9 @@ class VoxelGeneratorPlugin {
 // ---------------------------------------------------------------------------------------------
 // Shared by both conv plugins: device weights (+ epilogue), dtype bookkeeping, GEMM dispatch
 // ---------------------------------------------------------------------------------------------
+#ifndef SESSD_TILE_CUT_MIN_WORK
+#define SESSD_TILE_CUT_MIN_WORK (32 * 32)
+#endif
 class ConvPluginBase {
   public:
     virtual ~ConvPluginBase();
@@ -84,8 +87,14 @@ class ConvPluginBase {
 
   protected:
     // gather-GEMM over the neighbour table nbr[K][max_voxels] (device), rows < *num_out
-    int runGemm(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* num_out,
-                hipStream_t stream);
+    int runGemm(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* tiles,
+                const int32_t* num_out, hipStream_t stream);
+    // whether a rulebook built by this layer gets equal-work tile cuts: worth two small launches when the
+    // GEMM runs on the matrix cores and is not tiny
+    bool wantTileCuts() const {
+        return weights_packed_dev_ != nullptr && !(flags_ & SESSD_FLAG_FORCE_VALU) &&
+               in_channel_ * out_channel_ >= SESSD_TILE_CUT_MIN_WORK;
+    }
     int exportRulebook(const int32_t* nbr, const int32_t* num_out, void* scratch,
                        int32_t* indice_pairs, uint32_t* indice_num, hipStream_t stream) const;
     int freeDevice();

@@ -171,6 +171,7 @@ struct SparseConv3dLayerPlugin::Layout {
     uint64_t* first_words;
     uint32_t* block_counts;
     void* export_scratch;
+    int32_t* tiles;  // equal-work tile cuts of the rulebook (tile_cut.hip); first word 0 = none
     int32_t* meta;
     uint32_t cap;
     int Kc;
@@ -204,6 +205,7 @@ SparseConv3dLayerPlugin::Layout SparseConv3dLayerPlugin::carve(void* workspace) 
     L.first_words = c.take<uint64_t>((size_t)L.n_blocks * 4);
     L.block_counts = c.take<uint32_t>((size_t)L.n_blocks);
     L.export_scratch = c.take<uint8_t>(export_scratch_bytes(kernel_volume_, max_voxels_));
+    L.tiles = reinterpret_cast<int32_t*>(c.take<uint8_t>(tile_cut_bytes(max_voxels_)));
     L.meta_offset = c.offset;
     L.meta = c.take<int32_t>(4);
     L.total = c.total();
@@ -346,6 +348,7 @@ void SparseConv3dLayerPlugin::collectFill(void* workspace, int32_t* out_coors, F
     const Layout L = carve(workspace);
     f.add(L.keys, (uint64_t)L.cap * 2, kEmpty);
     f.add(L.nbr, (uint64_t)kernel_volume_ * max_voxels_, kEmpty);  // -1 = no input at this offset
+    f.add(L.tiles, 4, 0);
     f.add(L.meta, 4, 0);
     if (!(flags_ & SESSD_FLAG_SKIP_PAD_ROWS)) f.add(out_coors, (uint64_t)max_voxels_ * 4, 0);  // :668
 }
@@ -379,6 +382,7 @@ int SparseConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* v
                        L.n_blocks, out_coors, out_num, L.meta);
     hipLaunchKernelGGL(sp_scatter, grid, block, 0, stream, voxel_num, P, t, L.cand, L.nbr);
     SESSD_HIP_TRY(hipGetLastError());
+    if (wantTileCuts()) SESSD_TRY(launch_tile_cuts(L.nbr, out_num, kernel_volume_, max_voxels_, L.tiles, stream));
     return SESSD_OK;
 }
 
@@ -386,7 +390,7 @@ int SparseConv3dLayerPlugin::enqueueGemm(const void* in_feat, void* out_feat, co
                                          const void* workspace, hipStream_t stream) {
     if (!in_feat || !out_feat || !out_num || !workspace) return fail(SESSD_E_INVALID, "sparseconv3d.gemm: null pointer");
     const Layout L = carve(const_cast<void*>(workspace));
-    return runGemm(in_feat, out_feat, L.nbr, out_num, stream);
+    return runGemm(in_feat, out_feat, L.nbr, L.tiles, out_num, stream);
 }
 
 int SparseConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,

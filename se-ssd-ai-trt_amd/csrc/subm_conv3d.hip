@@ -80,6 +80,7 @@ struct SubmConv3dLayerPlugin::Layout {
     uint32_t* vals;
     int32_t* nbr;
     void* export_scratch;
+    int32_t* tiles;  // equal-work tile cuts of the rulebook (tile_cut.hip); first word 0 = none
     int32_t* meta;  // [0] status word, [1] active rows of the last enqueue
     uint32_t cap;
     size_t meta_offset;
@@ -94,6 +95,7 @@ SubmConv3dLayerPlugin::Layout SubmConv3dLayerPlugin::carve(void* workspace) cons
     L.vals = L.keys ? L.keys + L.cap : nullptr;
     L.nbr = c.take<int32_t>((size_t)kernel_volume_ * max_voxels_);
     L.export_scratch = c.take<uint8_t>(export_scratch_bytes(kernel_volume_, max_voxels_));
+    L.tiles = reinterpret_cast<int32_t*>(c.take<uint8_t>(tile_cut_bytes(max_voxels_)));
     L.meta_offset = c.offset;
     L.meta = c.take<int32_t>(4);
     L.total = c.total();
@@ -226,6 +228,7 @@ size_t SubmConv3dLayerPlugin::statusOffset() const { return carve(nullptr).meta_
 void SubmConv3dLayerPlugin::collectFill(void* workspace, FillArgs& f) const {
     const Layout L = carve(workspace);
     f.add(L.keys, (uint64_t)L.cap * 2, kEmpty);
+    f.add(L.tiles, 4, 0);
     f.add(L.meta, 4, 0);
 }
 
@@ -246,6 +249,7 @@ int SubmConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* vox
     hipLaunchKernelGGL(subm_neighbours, dim3(row_blocks, kernel_volume_), dim3(kBlock), 0, stream, coors,
                        voxel_num, max_voxels_, g, ksize_, padding_, t, L.nbr);
     SESSD_HIP_TRY(hipGetLastError());
+    if (wantTileCuts()) SESSD_TRY(launch_tile_cuts(L.nbr, voxel_num, kernel_volume_, max_voxels_, L.tiles, stream));
     return SESSD_OK;
 }
 
@@ -254,7 +258,7 @@ int SubmConv3dLayerPlugin::enqueueGemm(const void* in_feat, void* out_feat, cons
     if (!in_feat || !out_feat || !voxel_num || !rulebook_workspace)
         return fail(SESSD_E_INVALID, "submconv3d.gemm: null pointer");
     const Layout L = carve(const_cast<void*>(rulebook_workspace));
-    return runGemm(in_feat, out_feat, L.nbr, voxel_num, stream);
+    return runGemm(in_feat, out_feat, L.nbr, L.tiles, voxel_num, stream);
 }
 
 int SubmConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,

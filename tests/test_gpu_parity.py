@@ -147,6 +147,44 @@ def test_subm_clustered_with_epilogue_and_pad_rows(cin, cout):
     assert_features_close(out, o_out, RTOL_FP32, "subm %d->%d" % (cin, cout))   # incl. pad rows = relu(shift)
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+def test_equal_work_tiles_with_dense_and_isolated_regions(dtype):
+    """A fully dense block (27 pairs per row) followed by isolated voxels (1 pair per row): the equal-work tile
+    cuts give the isolated stretch runs far longer than the kernel's tile capacity, which it walks in pieces.
+    Shuffled row order as a second case (every tile mixes both kinds)."""
+    grid = (21, 800, 704)
+    rng = np.random.default_rng(31)
+    z, y, x = np.meshgrid(np.arange(2, 14), np.arange(100, 114), np.arange(200, 214), indexing="ij")
+    dense = np.stack([np.zeros(z.size, np.int64), z.ravel(), y.ravel(), x.ravel()], 1)
+    iso = np.stack([np.zeros(4000, np.int64), rng.integers(0, 21, 4000) // 3 * 3, 300 + 3 * (np.arange(4000) // 60),
+                    3 * (np.arange(4000) % 60)], 1)
+    iso = np.unique(iso, axis=0)
+    for order in ("blocked", "shuffled"):
+        coors = np.concatenate([dense, iso]).astype(np.int32)
+        if order == "shuffled":
+            coors = coors[rng.permutation(len(coors))]
+        n, mv = len(coors), 8192
+        feat = rng.uniform(-1, 1, (n, 64)).astype(np.float32)
+        w = rng.normal(0, 0.05, (27, 64, 64)).astype(np.float32)
+        o_pairs, o_num, _ = O.subm_rulebook(coors, n, grid[::-1], mv)
+        assert o_num[13] == n and int(o_num.sum()) > 20 * len(dense)
+        if dtype == "fp32":
+            conv, out, pairs, num, _ = run_subm(coors, n, feat, w, grid, mv)
+            assert np.array_equal(num, o_num)
+            assert_features_close(out[:n], O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv)[:n], RTOL_FP32, order)
+        else:
+            conv = api.SubmConv3d(64, 64, grid[::-1], w, mv)
+            cbuf = np.zeros((mv, 4), np.int32)
+            cbuf[:n] = coors
+            fbuf = np.zeros((mv, 64), np.float16)
+            fbuf[:n] = feat
+            out = to_np(conv(dev(fbuf), dev(cbuf), dev(np.array([n], np.int32))).float())
+            wh = w.astype(np.float16).astype(np.float32)
+            want = O.gather_gemm_scatter(fbuf[:n].astype(np.float32), wh, o_pairs, o_num, mv)[:n]
+            assert_features_close(out[:n], want, RTOL_FP16, order)
+        assert conv.status() == 0
+
+
 def test_mfma_and_valu_paths_agree():
     """The matrix-core kernel against the shape-agnostic VALU kernel on the same rulebook (both FP32)."""
     grid = (11, 120, 120)
