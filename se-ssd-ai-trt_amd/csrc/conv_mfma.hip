@@ -10,8 +10,9 @@
 //     with wave64 ballot + popcount: pair list k = the (input row, local output row) pairs of the rows
 //     that really have a neighbour at offset k.  Only those rows enter an MFMA block, so the matrix
 //     cores do not multiply the zero rows a dense [rows x K*Cin] gather matrix would be half full of.
-//   * Non-empty offsets are dealt round-robin to the four waves (split-K over offsets): tiles x 4 waves
-//     is what fills 256 CUs with a ~17k-row problem.
+//   * Non-empty offsets are dealt to the four waves, longest pair list first, each to the wave with the
+//     least work so far (split-K over offsets): tiles x 4 waves is what fills 256 CUs with a ~17k-row
+//     problem.
 //   * A wave gathers 16 pairs per MFMA block straight into operand registers: lane (i = lane%16,
 //     q = lane/16) loads 16 bytes of pair i's input row per K-chunk (FP32: channels 16g+4q..+3, FP16:
 //     channels 32g+8q..+7), i.e. every row is read as 64-byte segments.  The weights were reordered on
@@ -181,15 +182,40 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
     for (int t = lane; t < rows * LDP / 4; t += 64) reinterpret_cast<float4*>(part)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
 
-    // offsets this wave handles: the non-empty ones, dealt round-robin (all wave-uniform)
+    // offsets this wave handles.  An offset costs one MFMA pass per 16 pairs, so the offsets are dealt
+    // longest first, each to the wave with the least work so far (wave-uniform scalar code, the same in
+    // all four waves): round-robin dealing left the busiest wave ~13 % above the mean.
+    // Narrow layers have too little work per tile to pay for the dealing loop: plain round-robin there.
     uint32_t my_mask = 0;
-    {
+    if constexpr (CIN * COUT < 64 * 64) {
         int live = 0;
         for (int k = 0; k < K; ++k)
             if (s_cnt[k] > 0) {
                 if ((live % kWaves) == wave) my_mask |= 1u << k;
                 ++live;
             }
+    } else {
+        const int c = lane < K ? s_cnt[lane] : 0;
+        const int b = (c + 15) >> 4;
+        int load[kWaves];
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) load[w] = 0;
+#pragma unroll
+        for (int size = kMaxBlk; size >= 1; --size) {
+            uint64_t m = __ballot(b == size);
+            while (m) {
+                const int k = __ffsll((unsigned long long)m) - 1;
+                m &= m - 1;
+                int best = 0;
+#pragma unroll
+                for (int w = 1; w < kWaves; ++w)
+                    if (load[w] < load[best]) best = w;
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w)
+                    if (w == best) load[w] += size;
+                if (best == wave) my_mask |= 1u << k;
+            }
+        }
     }
 
     // gathered rows of all blocks of offset k -> operand registers (zeros for the padding pairs)
