@@ -28,7 +28,10 @@ struct GemmArgs {
 // r = the smallest tiles-per-CU count that keeps the mean tile at or below the target height, so that every
 // CU gets the same number of tiles (a fixed 32-row tiling leaves e.g. 529 tiles for 256 CUs: some CUs run
 // three tiles, most two, and the kernel lasts as long as the three).
-constexpr int kGemmTargetRows = 40;
+#ifndef SESSD_GEMM_TARGET_ROWS
+#define SESSD_GEMM_TARGET_ROWS 40
+#endif
+constexpr int kGemmTargetRows = SESSD_GEMM_TARGET_ROWS;
 struct TilePlan {
     int count;   // tiles
     int height;  // rows per tile when all tiles have the same length
