@@ -105,8 +105,12 @@ __device__ __forceinline__ void store4(__half* dst, const float (&o)[4]) {
     *reinterpret_cast<uint2*>(dst) = p.u;
 }
 
+// waves per SIMD the register allocation must leave room for: two workgroups per CU in the wide layers
+// (whose tiles come two to a CU), more in the narrow ones
+constexpr int min_waves_per_simd(int cin, int cout) { return cin * cout >= 32 * 64 ? 2 : (cin * cout >= 32 * 32 ? 3 : 4); }
+
 template <typename T, int CIN, int COUT>
-__global__ void __launch_bounds__(kWaves * 64)
+__global__ void __launch_bounds__(kWaves * 64, min_waves_per_simd(CIN, COUT))
 conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict__ Wp,
           const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
           const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad,
@@ -122,12 +126,25 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
     __shared__ int32_t s_cnt[kMaxK + 5];          // pairs per offset
     __shared__ float s_part[kWaves * kTileRows * LDP];
 
+    // the row count and the tile cuts are independent loads: request them together (a grid of
+    // tile_plan(max_voxels).count workgroups never indexes past the cut table)
     int n = *num_out;
+    const int cut_count = tiles ? tiles[0] : 0;
+    const int cut_begin = tiles ? tiles[4 + blockIdx.x] : 0;
+    const int cut_end = tiles ? tiles[5 + blockIdx.x] : 0;
     n = n < 0 ? 0 : (n > max_voxels ? max_voxels : n);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     constexpr int kVecPerRow = COUT / 4;
+    // scale/shift are fetched now, into LDS, so that the epilogue does not wait for global memory
+    __shared__ float s_epi[2 * COUT];
+    for (int c = tid; c < COUT; c += kWaves * 64) {
+        s_epi[c] = scale ? scale[c] : 1.f;
+        s_epi[COUT + c] = shift ? shift[c] : 0.f;
+    }
+    const int ec4 = (tid % kVecPerRow) * 4;  // this thread's epilogue columns, the same for every row it stores
+    static_assert((kWaves * 64) % kVecPerRow == 0, "a thread must keep its columns from row to row");
 
     // rows >= n: the reference zero-fills them (then BN+ReLU): epilogue(0), spread over all workgroups
     if (write_pad) {
@@ -150,10 +167,10 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
     }
     // this workgroup's run of rows: from the rulebook's equal-work cuts, or equal lengths
     int run_begin, run_end;
-    if (tiles && tiles[0] > 0) {
-        if ((int)blockIdx.x >= tiles[0]) return;
-        run_begin = tiles[4 + blockIdx.x];
-        run_end = tiles[5 + blockIdx.x];
+    if (cut_count > 0) {
+        if ((int)blockIdx.x >= cut_count) return;
+        run_begin = cut_begin;
+        run_end = cut_end;
     } else {
         const int R = tile_plan(n, num_cu).height;
         run_begin = blockIdx.x * R;
@@ -167,8 +184,19 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
     const int rows = run_end - row0 < kTileRows ? run_end - row0 : kTileRows;
 
     // ---- stage + compact: a wave turns one offset's neighbour list into a pair list per step ----
-    for (int k = wave; k < K; k += kWaves) {
-        const int v = lane < rows ? nbr[(size_t)k * max_voxels + row0 + lane] : -1;
+    // (all of a wave's list loads are requested before the first one is consumed)
+    constexpr int kListsPerWave = (kMaxK + kWaves - 1) / kWaves;
+    int staged[kListsPerWave];
+#pragma unroll
+    for (int s = 0; s < kListsPerWave; ++s) {
+        const int k = wave + s * kWaves;
+        staged[s] = (k < K && lane < rows) ? nbr[(size_t)k * max_voxels + row0 + lane] : -1;
+    }
+#pragma unroll
+    for (int s = 0; s < kListsPerWave; ++s) {
+        const int k = wave + s * kWaves;
+        if (k >= K) break;
+        const int v = staged[s];
         const uint64_t m = __ballot(v >= 0);
         if (v >= 0) {
             const int j = __popcll(m & ((1ull << lane) - 1ull));
@@ -182,40 +210,24 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
     for (int t = lane; t < rows * LDP / 4; t += 64) reinterpret_cast<float4*>(part)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
 
-    // offsets this wave handles.  An offset costs one MFMA pass per 16 pairs, so the offsets are dealt
-    // longest first, each to the wave with the least work so far (wave-uniform scalar code, the same in
-    // all four waves): round-robin dealing left the busiest wave ~13 % above the mean.
-    // Narrow layers have too little work per tile to pay for the dealing loop: plain round-robin there.
-    uint32_t my_mask = 0;
-    if constexpr (CIN * COUT < 64 * 64) {
-        int live = 0;
-        for (int k = 0; k < K; ++k)
-            if (s_cnt[k] > 0) {
-                if ((live % kWaves) == wave) my_mask |= 1u << k;
-                ++live;
-            }
-    } else {
+    // offsets this wave handles.  An offset costs one MFMA pass per 16 pairs, so the offsets are ranked by
+    // pass count (ballots: lane k holds offset k) and dealt in that order back and forth over the waves
+    // (0 1 2 3 3 2 1 0 ...): plain round-robin left the busiest wave ~13 % above the mean, this ~8 %.
+    uint32_t my_mask;
+    {
         const int c = lane < K ? s_cnt[lane] : 0;
         const int b = (c + 15) >> 4;
-        int load[kWaves];
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) load[w] = 0;
+        const uint64_t below = (1ull << lane) - 1ull;
+        int rank = 0, ahead = 0;
 #pragma unroll
         for (int size = kMaxBlk; size >= 1; --size) {
-            uint64_t m = __ballot(b == size);
-            while (m) {
-                const int k = __ffsll((unsigned long long)m) - 1;
-                m &= m - 1;
-                int best = 0;
-#pragma unroll
-                for (int w = 1; w < kWaves; ++w)
-                    if (load[w] < load[best]) best = w;
-#pragma unroll
-                for (int w = 0; w < kWaves; ++w)
-                    if (w == best) load[w] += size;
-                if (best == wave) my_mask |= 1u << k;
-            }
+            const uint64_t m = __ballot(b == size);
+            if (b == size) rank = ahead + __popcll(m & below);
+            ahead += __popcll(m);
         }
+        const int r8 = rank & (2 * kWaves - 1);
+        const int w = r8 < kWaves ? r8 : 2 * kWaves - 1 - r8;
+        my_mask = (uint32_t)__ballot(b > 0 && w == wave);
     }
 
     // gathered rows of all blocks of offset k -> operand registers (zeros for the padding pairs)
@@ -303,19 +315,26 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
 
     // fixed-order sum of the four partials, epilogue, coalesced stores
     for (int v = tid; v < rows * kVecPerRow; v += kWaves * 64) {
-        const int r = v / kVecPerRow, c4 = (v % kVecPerRow) * 4;
-        float o[4];
+        const int r = v / kVecPerRow;
+        float4 acc4 = *reinterpret_cast<const float4*>(s_part + (0 * kTileRows + r) * LDP + ec4);
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) {
+            const float4 p4 = *reinterpret_cast<const float4*>(s_part + (w * kTileRows + r) * LDP + ec4);
+            acc4.x += p4.x;
+            acc4.y += p4.y;
+            acc4.z += p4.z;
+            acc4.w += p4.w;
+        }
+        float o[4] = {acc4.x, acc4.y, acc4.z, acc4.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            float s = s_part[(0 * kTileRows + r) * LDP + c4 + e];
-#pragma unroll
-            for (int w = 1; w < kWaves; ++w) s += s_part[(w * kTileRows + r) * LDP + c4 + e];
-            if (scale) s = s * scale[c4 + e];
-            if (shift) s = s + shift[c4 + e];
+            float s = o[e];
+            if (scale) s = s * s_epi[ec4 + e];
+            if (shift) s = s + s_epi[COUT + ec4 + e];
             if (relu) s = s > 0.f ? s : 0.f;
             o[e] = s;
         }
-        store4(out + (size_t)(row0 + r) * COUT + c4, o);
+        store4(out + (size_t)(row0 + r) * COUT + ec4, o);
     }
     __syncthreads();  // the next piece reuses the lists and partial tiles
     }
