@@ -107,7 +107,9 @@ __device__ __forceinline__ void store4(__half* dst, const float (&o)[4]) {
 
 // waves per SIMD the register allocation must leave room for: two workgroups per CU in the wide layers
 // (whose tiles come two to a CU), more in the narrow ones
-constexpr int min_waves_per_simd(int cin, int cout) { return cin * cout >= 32 * 64 ? 2 : (cin * cout >= 32 * 32 ? 3 : 4); }
+constexpr int min_waves_per_simd(int cin, int cout) {
+    return cout >= 128 ? 1 : (cin * cout >= 32 * 64 ? 2 : (cin * cout >= 32 * 32 ? 3 : 4));
+}
 
 template <typename T, int CIN, int COUT>
 __global__ void __launch_bounds__(kWaves * 64, min_waves_per_simd(CIN, COUT))
@@ -257,7 +259,7 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
     Vec a_cur[kMaxBlk][G], a_nxt[kMaxBlk][G], b[G][NB];
     int cnt_cur = 0, cnt_nxt = 0;
     if (k_cur >= 0) {
-        cnt_cur = s_cnt[k_cur];
+        cnt_cur = __builtin_amdgcn_readfirstlane(s_cnt[k_cur]);
         load_a(k_cur, cnt_cur, a_cur);
 #pragma unroll
         for (int g = 0; g < G; ++g) load_b(k_cur, g, b[g]);
@@ -266,7 +268,7 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
         const int k_nxt = my_mask ? __ffs(my_mask) - 1 : -1;
         my_mask &= my_mask - 1;
         if (k_nxt >= 0) {
-            cnt_nxt = s_cnt[k_nxt];
+            cnt_nxt = __builtin_amdgcn_readfirstlane(s_cnt[k_nxt]);  // wave-uniform: keep it scalar
             load_a(k_nxt, cnt_nxt, a_nxt);
         }
         v4f acc[kMaxBlk][NB];
