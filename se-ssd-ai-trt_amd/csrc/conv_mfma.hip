@@ -47,7 +47,7 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 constexpr int kWaves = SESSD_MFMA_WAVES;
 constexpr int kTileRows = SESSD_MFMA_TM;        // capacity: most output rows a workgroup can own (<= 64)
 constexpr int kMaxBlk = (kTileRows + 15) / 16;  // MFMA row blocks an offset can need
-constexpr int kMaxK = 27;
+constexpr int kMaxK = kGemmMaxOffsets;
 
 static_assert(kGemmTargetRows <= kTileRows && kTileRows <= 64, "tile height must fit the capacity and one wave");
 

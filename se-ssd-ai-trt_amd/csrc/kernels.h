@@ -32,6 +32,7 @@ struct GemmArgs {
 #define SESSD_GEMM_TARGET_ROWS 40
 #endif
 constexpr int kGemmTargetRows = SESSD_GEMM_TARGET_ROWS;
+constexpr int kGemmMaxOffsets = 27;  // kernel volumes the rulebook holds (3 x 3 x 3)
 struct TilePlan {
     int count;   // tiles
     int height;  // rows per tile when all tiles have the same length

@@ -39,8 +39,13 @@ tile_weights(const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_ou
     const int row = blockIdx.x * kBlock + threadIdx.x;
     int v = 0;
     if (row < n) {
+        // all K loads of the thread are requested before the first is used
+        int32_t e[kGemmMaxOffsets];
+#pragma unroll
+        for (int k = 0; k < kGemmMaxOffsets; ++k) e[k] = k < K ? nbr[(size_t)k * max_voxels + row] : -1;
         v = kRowWeight;
-        for (int k = 0; k < K; ++k) v += nbr[(size_t)k * max_voxels + row] >= 0 ? 1 : 0;
+#pragma unroll
+        for (int k = 0; k < kGemmMaxOffsets; ++k) v += e[k] >= 0 ? 1 : 0;
     }
     if (row < max_voxels) w[row] = v;
     int s = v;
