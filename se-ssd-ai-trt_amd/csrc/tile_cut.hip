@@ -30,28 +30,42 @@ constexpr int kRowWeight = SESSD_TILE_ROW_WEIGHT;
 
 __host__ __device__ inline int max_tiles(int max_voxels) { return max_voxels / kGemmTargetRows + 1024 + 1; }
 
-__global__ void __launch_bounds__(kBlock)
+// 256 rows per block, four threads per row (each sums every fourth offset): 1024 threads
+constexpr int kSplit = 4;
+__global__ void __launch_bounds__(kBlock * kSplit)
 tile_weights(const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
              int32_t* __restrict__ w, int32_t* __restrict__ bsum) {
+    __shared__ int32_t s_cnt[kSplit][kBlock];
     __shared__ int32_t s_part[kBlock / 64];
     int n = *num_out;
     n = n < 0 ? 0 : (n > max_voxels ? max_voxels : n);
-    const int row = blockIdx.x * kBlock + threadIdx.x;
-    int v = 0;
+    const int r = threadIdx.x % kBlock, kg = threadIdx.x / kBlock;
+    const int row = blockIdx.x * kBlock + r;
+    int c = 0;
     if (row < n) {
-        // all K loads of the thread are requested before the first is used
-        int32_t e[kGemmMaxOffsets];
+        constexpr int kPer = (kGemmMaxOffsets + kSplit - 1) / kSplit;
+        int32_t e[kPer];  // all loads of the thread are requested before the first is used
 #pragma unroll
-        for (int k = 0; k < kGemmMaxOffsets; ++k) e[k] = k < K ? nbr[(size_t)k * max_voxels + row] : -1;
+        for (int j = 0; j < kPer; ++j) {
+            const int k = kg + j * kSplit;
+            e[j] = k < K ? nbr[(size_t)k * max_voxels + row] : -1;
+        }
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) c += e[j] >= 0 ? 1 : 0;
+    }
+    s_cnt[kg][r] = c;
+    __syncthreads();
+    int v = 0;
+    if (kg == 0 && row < n) {
         v = kRowWeight;
 #pragma unroll
-        for (int k = 0; k < kGemmMaxOffsets; ++k) v += e[k] >= 0 ? 1 : 0;
+        for (int g = 0; g < kSplit; ++g) v += s_cnt[g][r];
     }
-    if (row < max_voxels) w[row] = v;
+    if (kg == 0 && row < max_voxels) w[row] = v;
     int s = v;
 #pragma unroll
     for (int d = 32; d > 0; d >>= 1) s += __shfl_xor(s, d, 64);
-    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = s;
+    if (kg == 0 && (r & 63) == 0) s_part[r >> 6] = s;
     __syncthreads();
     if (threadIdx.x == 0) bsum[blockIdx.x] = s_part[0] + s_part[1] + s_part[2] + s_part[3];
 }
@@ -126,7 +140,7 @@ int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_
     int32_t* w = hdr + 4 + max_tiles(max_voxels) + 1;
     int32_t* bsum = w + max_voxels;
     const int blocks = ceil_div(max_voxels, kBlock);
-    hipLaunchKernelGGL(tile_weights, dim3(blocks), dim3(kBlock), 0, stream, nbr, num_out, max_voxels, K, w, bsum);
+    hipLaunchKernelGGL(tile_weights, dim3(blocks), dim3(kBlock * kSplit), 0, stream, nbr, num_out, max_voxels, K, w, bsum);
     hipLaunchKernelGGL(tile_cuts, dim3(blocks), dim3(kBlock), 0, stream, num_out, max_voxels, gemm_compute_units(), w,
                        bsum, hdr);
     SESSD_HIP_TRY(hipGetLastError());
