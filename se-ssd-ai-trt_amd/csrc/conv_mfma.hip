@@ -69,6 +69,18 @@ struct Chunk<float, CIN> {
     }
 };
 
+// Cin = 4 (the voxel means entering the first layer): the whole inner dimension of an offset is one MFMA
+// K-step, a lane holds a single channel
+template <>
+struct Chunk<float, 4> {
+    using Vec = float;
+    static constexpr int kChannels = 4, kLaneElems = 1;
+    static __device__ __forceinline__ Vec zero() { return 0.f; }
+    static __device__ __forceinline__ void mma(const Vec& w, const Vec& x, v4f& acc) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w, x, acc, 0, 0, 0);
+    }
+};
+
 template <int CIN>
 struct Chunk<__half, CIN> {
     using Vec = float4;  // 8 halfs = channels 32g+8q .. +7
@@ -367,8 +379,9 @@ int launch(const GemmArgs& a, hipStream_t stream) {
     return SESSD_OK;
 }
 
-bool mfma_shape(int K, int cin, int cout) {
+bool mfma_shape(int K, int cin, int cout, int dtype) {
     if (K > kMaxK) return false;
+    if (cin == 4) return dtype == SESSD_FLOAT && (cout == 16 || cout == 32);
     const int shapes[][2] = {{16, 16}, {16, 32}, {32, 32}, {32, 64}, {64, 64}, {64, 128}, {128, 128}};
     for (auto& s : shapes)
         if (s[0] == cin && s[1] == cout) return true;
@@ -377,7 +390,10 @@ bool mfma_shape(int K, int cin, int cout) {
 
 // channels per K-chunk and elements per lane, as in Chunk<>
 void chunk_shape(int dtype, int cin, int* channels, int* lane_elems) {
-    if (dtype == SESSD_FLOAT) {
+    if (dtype == SESSD_FLOAT && cin == 4) {
+        *channels = 4;
+        *lane_elems = 1;
+    } else if (dtype == SESSD_FLOAT) {
         *channels = 16;
         *lane_elems = 4;
     } else if (cin == 16) {
@@ -394,7 +410,7 @@ void chunk_shape(int dtype, int cin, int* channels, int* lane_elems) {
 int gemm_compute_units() { return compute_units(); }
 
 size_t packed_weight_bytes(int K, int cin, int cout, int dtype) {
-    if (!mfma_shape(K, cin, cout)) return 0;
+    if (!mfma_shape(K, cin, cout, dtype)) return 0;
     return (size_t)K * cin * cout * (dtype == SESSD_HALF ? sizeof(__half) : sizeof(float));
 }
 
@@ -418,12 +434,14 @@ void pack_weights(const float* w, int K, int cin, int cout, int dtype, void* dst
 
 // -> SESSD_OK when an MFMA kernel was launched, SESSD_E_UNSUPPORTED when the shape/dtype is not covered
 int launch_mfma(const GemmArgs& a, hipStream_t stream) {
-    if (a.in_type != a.out_type || !a.w_packed || !mfma_shape(a.K, a.cin, a.cout)) return SESSD_E_UNSUPPORTED;
+    if (a.in_type != a.out_type || !a.w_packed || !mfma_shape(a.K, a.cin, a.cout, a.in_type)) return SESSD_E_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(a.in_feat) | reinterpret_cast<uintptr_t>(a.out_feat)) & 15)
         return SESSD_E_UNSUPPORTED;
 #define SESSD_CASE(CI, CO)                                                        \
     if (a.cin == CI && a.cout == CO)                                              \
     return a.in_type == SESSD_HALF ? launch<__half, CI, CO>(a, stream) : launch<float, CI, CO>(a, stream)
+    if (a.cin == 4 && a.cout == 16) return launch<float, 4, 16>(a, stream);  // (FP32 only: mfma_shape)
+    if (a.cin == 4 && a.cout == 32) return launch<float, 4, 32>(a, stream);
     SESSD_CASE(16, 16);
     SESSD_CASE(16, 32);
     SESSD_CASE(32, 32);
