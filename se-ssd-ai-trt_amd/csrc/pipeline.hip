@@ -125,16 +125,31 @@ struct Pipeline {
         SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_fill, 0));
         const int32_t* coors = static_cast<const int32_t*>(vg_coors.p);
         const int32_t* num = static_cast<const int32_t*>(vg_num.p);
+        // The kernel that produced a coors tensor has left a cell -> row hash behind (the voxelizer's, or a
+        // strided layer's): a SubM layer on the same grid looks its neighbours up in that table and skips its
+        // own insert pass.  `cells` = that table, {cx, cy, cz} = the x/y grid it is keyed on and its z extent.
+        HashTable cells = vg->cellTable(vg_ws.p, desc.max_points);
+        int cx = vg->grid_x_size_, cy = vg->grid_y_size_, cz = vg->grid_z_size_;
         for (size_t l = 0; l < stages.size(); ++l) {
             ConvStage& st = *stages[l];
             if (st.subm) {
                 if (st.rulebook_from >= 0) continue;
-                SESSD_TRY(st.subm->enqueueBuild(coors, num, st.ws.p, aux, true));
+                // keys are (z*Y + y)*X + x: the same number in both grids when X and Y agree; cells of the
+                // layer's grid beyond the table's z extent are simply absent
+                // (a strided layer's table is sized for every candidate cell of max_voxels inputs; beyond 2^20
+                // slots -- 4 MB of keys, one XCD's L2 -- probing it costs more than the insert pass it saves)
+                const bool same_grid = st.subm->out_shape_x_ == cx && st.subm->out_shape_y_ == cy &&
+                                       st.subm->out_shape_z_ >= cz && cells.mask < (1u << 20);
+                SESSD_TRY(st.subm->enqueueBuild(coors, num, st.ws.p, aux, true, same_grid ? &cells : nullptr));
             } else {
                 SESSD_TRY(st.sparse->enqueueBuild(coors, num, static_cast<int32_t*>(st.coors.p),
                                                   static_cast<int32_t*>(st.num.p), st.ws.p, aux, true));
                 coors = static_cast<const int32_t*>(st.coors.p);
                 num = static_cast<const int32_t*>(st.num.p);
+                cells = st.sparse->cellTable(st.ws.p);
+                cx = st.sparse->out_shape_x_;
+                cy = st.sparse->out_shape_y_;
+                cz = st.sparse->out_shape_z_;
             }
             SESSD_HIP_TRY(hipEventRecord(ev_build[l], aux));
         }

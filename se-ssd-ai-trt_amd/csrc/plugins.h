@@ -34,6 +34,10 @@ class VoxelGeneratorPlugin {
     size_t getSerializationSize() const;
     void serialize(void* buffer) const;
     size_t statusOffset(int max_points) const;
+    // After an enqueue the workspace's hash maps linear cell (z*Y + y)*X + x -> voxel row (kEmpty for cells
+    // dropped at the cap): a SubM layer on the same x/y grid can use it as its cell table
+    // (SubmConv3dLayerPlugin::enqueueBuild) instead of inserting every voxel into its own.
+    HashTable cellTable(void* workspace, int max_points) const;
 
     // serialized fields, in the reference's order (voxelGenerator.cu:584-599)
     int voxelNum_ = 0;      // max_voxels
@@ -121,8 +125,10 @@ class SubmConv3dLayerPlugin : public ConvPluginBase {
                       const void* const* inputs, void* const* outputs,
                       const void* rulebook_workspace, hipStream_t stream);
     // enqueue = enqueueBuild (coordinates -> rulebook) + enqueueGemm (features)
+    // `cells`: a cell -> row table over this layer's grid that some earlier kernel already built (the
+    // voxelizer's, or that of the strided layer that produced `coors`); the insert pass is skipped then
     int enqueueBuild(const int32_t* coors, const int32_t* voxel_num, void* workspace, hipStream_t stream,
-                     bool prefilled = false);
+                     bool prefilled = false, const HashTable* cells = nullptr);
     void collectFill(void* workspace, FillArgs& f) const;
     int enqueueGemm(const void* in_feat, void* out_feat, const int32_t* voxel_num,
                     const void* rulebook_workspace, hipStream_t stream);
@@ -162,6 +168,8 @@ class SparseConv3dLayerPlugin : public ConvPluginBase {
     int countPairs(const void* workspace, uint32_t* indice_num, hipStream_t stream) const;
     int enqueueBuild(const int32_t* coors, const int32_t* voxel_num, int32_t* out_coors, int32_t* out_num,
                      void* workspace, hipStream_t stream, bool prefilled = false);
+    // after enqueueBuild the workspace's hash maps output cell -> output row (see VoxelGeneratorPlugin::cellTable)
+    HashTable cellTable(void* workspace) const;
     void collectFill(void* workspace, int32_t* out_coors, FillArgs& f) const;
     int enqueueGemm(const void* in_feat, void* out_feat, const int32_t* out_num, const void* workspace,
                     hipStream_t stream);

@@ -386,6 +386,11 @@ int SparseConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* v
     return SESSD_OK;
 }
 
+HashTable SparseConv3dLayerPlugin::cellTable(void* workspace) const {
+    const Layout L = carve(workspace);
+    return make_hash(L.keys, L.vals, L.cap);
+}
+
 int SparseConv3dLayerPlugin::enqueueGemm(const void* in_feat, void* out_feat, const int32_t* out_num,
                                          const void* workspace, hipStream_t stream) {
     if (!in_feat || !out_feat || !out_num || !workspace) return fail(SESSD_E_INVALID, "sparseconv3d.gemm: null pointer");

@@ -55,10 +55,11 @@ subm_insert(const int32_t* __restrict__ coors, const int32_t* __restrict__ voxel
 // cell i sits at o - padding + k on every axis (stride 1, dilation 1).
 __global__ void __launch_bounds__(kBlock)
 subm_neighbours(const int32_t* __restrict__ coors, const int32_t* __restrict__ voxel_num, int max_voxels,
-                Grid3 g, int ksize, int padding, HashTable t, int32_t* __restrict__ nbr) {
+                Grid3 g, int ksize, int padding, HashTable t, int32_t* __restrict__ nbr, int32_t* meta) {
     const int v = blockIdx.x * kBlock + threadIdx.x;
     const int k = blockIdx.y;
     const int n = clamp_count(voxel_num, max_voxels);
+    if (meta && v == 0 && k == 0) meta[1] = n;  // (subm_insert's job when that pass runs)
     if (v >= n) return;
     const int4 c = reinterpret_cast<const int4*>(coors)[v];
     const int kz = k / (ksize * ksize), ky = (k / ksize) % ksize, kx = k % ksize;
@@ -233,7 +234,7 @@ void SubmConv3dLayerPlugin::collectFill(void* workspace, FillArgs& f) const {
 }
 
 int SubmConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* voxel_num, void* workspace,
-                                        hipStream_t stream, bool prefilled) {
+                                        hipStream_t stream, bool prefilled, const HashTable* cells) {
     if (!coors || !voxel_num || !workspace) return fail(SESSD_E_INVALID, "submconv3d.build: null pointer");
     const Layout L = carve(workspace);
     const HashTable t = make_hash(L.keys, L.vals, L.cap);
@@ -244,10 +245,12 @@ int SubmConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* vox
         SESSD_TRY(launch_fill(f, stream));
     }
     const int row_blocks = ceil_div(max_voxels_, kBlock);
-    hipLaunchKernelGGL(subm_insert, dim3(row_blocks), dim3(kBlock), 0, stream, coors, voxel_num, max_voxels_,
-                       g, t, L.meta);
+    if (!cells)
+        hipLaunchKernelGGL(subm_insert, dim3(row_blocks), dim3(kBlock), 0, stream, coors, voxel_num, max_voxels_,
+                           g, t, L.meta);
     hipLaunchKernelGGL(subm_neighbours, dim3(row_blocks, kernel_volume_), dim3(kBlock), 0, stream, coors,
-                       voxel_num, max_voxels_, g, ksize_, padding_, t, L.nbr);
+                       voxel_num, max_voxels_, g, ksize_, padding_, cells ? *cells : t, L.nbr,
+                       cells ? L.meta : nullptr);
     SESSD_HIP_TRY(hipGetLastError());
     if (wantTileCuts()) SESSD_TRY(launch_tile_cuts(L.nbr, voxel_num, kernel_volume_, max_voxels_, L.tiles, stream));
     return SESSD_OK;

@@ -140,6 +140,7 @@ vg_finalize(const float* __restrict__ points, int pf, VgParams p, HashTable t,
     const int iy = rem / p.gx;
     const int ix = rem - iy * p.gx;
     reinterpret_cast<int4*>(coors)[vid] = make_int4(0, iz, iy, ix);  // voxelGenerator.cu:404-405
+    t.vals[slot] = vid;  // the table now maps cell -> voxel row (VoxelGeneratorPlugin::cellTable)
 
     // voxelGenerator.cu:274-296: all S slots are summed left to right, unfilled slots count as 0
     const uint32_t* s = slots + (size_t)slot * p.max_pts;
@@ -171,6 +172,7 @@ int np_round(float x) {
 
 struct VoxelGeneratorPlugin::Layout {
     uint32_t* keys;
+    uint32_t* vals;  // voxel row of the cell (written by vg_finalize; kEmpty for dropped cells)
     uint32_t* slots;
     int32_t* pt_slot;
     uint64_t* first_words;
@@ -187,10 +189,12 @@ VoxelGeneratorPlugin::Layout VoxelGeneratorPlugin::carve(void* workspace, int ma
     WorkspaceCarver c(workspace);
     L.cap = next_pow2((uint64_t)(max_points < 32 ? 32 : max_points) * 2);
     L.n_blocks = ceil_div(max_points, kBlock);
-    // keys and slots are adjacent so that one fill region clears both
-    const size_t table_words = align_up((size_t)L.cap * 4) / 4 + (size_t)L.cap * pointNum_;
+    // keys, vals and slots are adjacent so that one fill region clears all three
+    const size_t cap_words = align_up((size_t)L.cap * 4) / 4;
+    const size_t table_words = 2 * cap_words + (size_t)L.cap * pointNum_;
     L.keys = c.take<uint32_t>(table_words);
-    L.slots = L.keys ? L.keys + align_up((size_t)L.cap * 4) / 4 : nullptr;
+    L.vals = L.keys ? L.keys + cap_words : nullptr;
+    L.slots = L.keys ? L.keys + 2 * cap_words : nullptr;
     L.pt_slot = c.take<int32_t>((size_t)L.n_blocks * kBlock);
     L.first_words = c.take<uint64_t>((size_t)L.n_blocks * 4);
     L.block_counts = c.take<uint32_t>((size_t)L.n_blocks);
@@ -198,6 +202,11 @@ VoxelGeneratorPlugin::Layout VoxelGeneratorPlugin::carve(void* workspace, int ma
     L.status = c.take<int32_t>(4);
     L.total = c.total();
     return L;
+}
+
+HashTable VoxelGeneratorPlugin::cellTable(void* workspace, int max_points) const {
+    const Layout L = carve(workspace, max_points);
+    return make_hash(L.keys, L.vals, L.cap);
 }
 
 void VoxelGeneratorPlugin::deriveGrid() {
@@ -336,7 +345,7 @@ int VoxelGeneratorPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sess
 
     lastMaxPoints_ = max_points;
     const Layout L = carve(workspace, max_points);
-    HashTable t = make_hash(L.keys, nullptr, L.cap);
+    HashTable t = make_hash(L.keys, L.vals, L.cap);
     VgParams p{min_x_range_, max_x_range_, min_y_range_, max_y_range_, min_z_range_, max_z_range_,
                voxel_x_size_, voxel_y_size_, voxel_z_size_, grid_x_size_, grid_y_size_, grid_z_size_,
                voxelNum_, pointNum_};
