@@ -120,7 +120,7 @@ __device__ __forceinline__ void store4(__half* dst, const float (&o)[4]) {
 // waves per SIMD the register allocation must leave room for: two workgroups per CU in the wide layers
 // (whose tiles come two to a CU), more in the narrow ones
 constexpr int min_waves_per_simd(int cin, int cout) {
-    return cout >= 128 ? 1 : (cin * cout >= 32 * 64 ? 2 : (cin * cout >= 32 * 32 ? 3 : 4));
+    return cin * cout >= 32 * 64 ? 2 : (cin * cout >= 32 * 32 ? 3 : 4);
 }
 
 template <typename T, int CIN, int COUT>
@@ -132,8 +132,16 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
     using C = Chunk<T, CIN>;
     using Vec = typename C::Vec;
     constexpr int G = CIN / C::kChannels;  // K-chunks of the inner dimension
-    constexpr int NB = COUT / 16;          // 16-column blocks
-    constexpr int LDP = COUT + 4;          // padded row stride of the partial tiles in LDS
+    constexpr int NBT = COUT / 16;         // 16-column blocks of the layer
+    // 128 output columns: the waves pair up, each wave of a pair takes half of the columns of the offsets
+    // dealt to the pair.  Weight registers, accumulators and the wave's partial tile then have the size of
+    // the 64-column case (two workgroups per CU instead of one wave per SIMD and 100 KB of LDS); the price
+    // is that both waves of a pair gather the rows of their offsets.
+    constexpr int CS = COUT >= 128 ? 2 : 1;  // waves sharing an offset (column split)
+    constexpr int KG = kWaves / CS;          // groups the offsets are dealt to
+    constexpr int NB = NBT / CS;             // column blocks of one wave
+    constexpr int CW = COUT / CS;            // columns of one wave
+    constexpr int LDP = CW + 4;              // padded row stride of the partial tiles in LDS
     static_assert(CIN % C::kChannels == 0 && COUT % 16 == 0, "channel counts must fill whole MFMA chunks");
     __shared__ int32_t s_in[kMaxK * kTileRows];   // compacted pair lists: input row ...
     __shared__ uint8_t s_row[kMaxK * kTileRows];  // ... and local output row of pair j of offset k
@@ -150,6 +158,8 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    const int kgrp = wave / CS;   // offsets are dealt to this group ...
+    const int chalf = wave % CS;  // ... and this wave computes this part of their columns
     constexpr int kVecPerRow = COUT / 4;
     // scale/shift are fetched now, into LDS, so that the epilogue does not wait for global memory
     __shared__ float s_epi[2 * COUT];
@@ -239,9 +249,9 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
             if (b == size) rank = ahead + __popcll(m & below);
             ahead += __popcll(m);
         }
-        const int r8 = rank & (2 * kWaves - 1);
-        const int w = r8 < kWaves ? r8 : 2 * kWaves - 1 - r8;
-        my_mask = (uint32_t)__ballot(b > 0 && w == wave);
+        const int r8 = rank % (2 * KG);
+        const int w = r8 < KG ? r8 : 2 * KG - 1 - r8;
+        my_mask = (uint32_t)__ballot(b > 0 && w == kgrp);
     }
 
     // gathered rows of all blocks of offset k -> operand registers (zeros for the padding pairs)
@@ -261,7 +271,7 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
         }
     };
     auto load_b = [&](int k, int g, Vec (&b)[NB]) {
-        const Vec* wk = wp + ((size_t)k * G + g) * NB * 64;
+        const Vec* wk = wp + (((size_t)k * G + g) * NBT + chalf * NB) * 64;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) b[nb] = wk[nb * 64];
     };
@@ -330,10 +340,12 @@ conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict_
     // fixed-order sum of the four partials, epilogue, coalesced stores
     for (int v = tid; v < rows * kVecPerRow; v += kWaves * 64) {
         const int r = v / kVecPerRow;
-        float4 acc4 = *reinterpret_cast<const float4*>(s_part + (0 * kTileRows + r) * LDP + ec4);
+        // the partial tiles of the KG waves that hold this column, in a fixed order
+        const float* col = s_part + ((ec4 / CW) * kTileRows + r) * LDP + ec4 % CW;
+        float4 acc4 = *reinterpret_cast<const float4*>(col);
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) {
-            const float4 p4 = *reinterpret_cast<const float4*>(s_part + (w * kTileRows + r) * LDP + ec4);
+        for (int w = 1; w < KG; ++w) {
+            const float4 p4 = *reinterpret_cast<const float4*>(col + w * CS * kTileRows * LDP);
             acc4.x += p4.x;
             acc4.y += p4.y;
             acc4.z += p4.z;
