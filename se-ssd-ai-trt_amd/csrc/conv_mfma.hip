@@ -123,9 +123,11 @@ constexpr int min_waves_per_simd(int cin, int cout) {
     return cin * cout >= 32 * 64 ? 2 : (cin * cout >= 32 * 32 ? 3 : 4);
 }
 
-template <typename T, int CIN, int COUT>
+// T = type of the input features and of the arithmetic's operands, TO = type the output rows are stored
+// in (differs only for the first layer of an FP16 pipeline: FP32 voxel means in, FP16 features out)
+template <typename T, int CIN, int COUT, typename TO = T>
 __global__ void __launch_bounds__(kWaves * 64, min_waves_per_simd(CIN, COUT))
-conv_mfma(const T* __restrict__ in, T* __restrict__ out, const void* __restrict__ Wp,
+conv_mfma(const T* __restrict__ in, TO* __restrict__ out, const void* __restrict__ Wp,
           const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
           const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad,
           int num_cu, const int32_t* __restrict__ tiles) {
@@ -379,13 +381,13 @@ int compute_units() {
     return cu;
 }
 
-template <typename T, int CIN, int COUT>
+template <typename T, int CIN, int COUT, typename TO = T>
 int launch(const GemmArgs& a, hipStream_t stream) {
     const int num_cu = compute_units();
     // tile_plan() never cuts n <= max_voxels rows into more tiles than it does max_voxels rows
     const unsigned blocks = (unsigned)tile_plan(a.max_voxels, num_cu).count;
-    hipLaunchKernelGGL((conv_mfma<T, CIN, COUT>), dim3(blocks), dim3(kWaves * 64), 0, stream,
-                       static_cast<const T*>(a.in_feat), static_cast<T*>(a.out_feat), a.w_packed, a.nbr,
+    hipLaunchKernelGGL((conv_mfma<T, CIN, COUT, TO>), dim3(blocks), dim3(kWaves * 64), 0, stream,
+                       static_cast<const T*>(a.in_feat), static_cast<TO*>(a.out_feat), a.w_packed, a.nbr,
                        a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows, num_cu, a.tiles);
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;
@@ -393,7 +395,7 @@ int launch(const GemmArgs& a, hipStream_t stream) {
 
 bool mfma_shape(int K, int cin, int cout, int dtype) {
     if (K > kMaxK) return false;
-    if (cin == 4) return dtype == SESSD_FLOAT && (cout == 16 || cout == 32);
+    if (cin == 4) return cout == 16 || cout == 32;  // FP32 operands whatever the pipeline's feature dtype
     const int shapes[][2] = {{16, 16}, {16, 32}, {32, 32}, {32, 64}, {64, 64}, {64, 128}, {128, 128}};
     for (auto& s : shapes)
         if (s[0] == cin && s[1] == cout) return true;
@@ -402,7 +404,7 @@ bool mfma_shape(int K, int cin, int cout, int dtype) {
 
 // channels per K-chunk and elements per lane, as in Chunk<>
 void chunk_shape(int dtype, int cin, int* channels, int* lane_elems) {
-    if (dtype == SESSD_FLOAT && cin == 4) {
+    if (cin == 4) {
         *channels = 4;
         *lane_elems = 1;
     } else if (dtype == SESSD_FLOAT) {
@@ -423,11 +425,13 @@ int gemm_compute_units() { return compute_units(); }
 
 size_t packed_weight_bytes(int K, int cin, int cout, int dtype) {
     if (!mfma_shape(K, cin, cout, dtype)) return 0;
-    return (size_t)K * cin * cout * (dtype == SESSD_HALF ? sizeof(__half) : sizeof(float));
+    return (size_t)K * cin * cout * (dtype == SESSD_HALF && cin != 4 ? sizeof(__half) : sizeof(float));
 }
 
 // Operand order: Wp[k][g][nb][lane][e] = W[k][C*g + E*(lane/16) + e][16nb + lane%16] with C channels per
-// K-chunk and E elements per lane (FP32: 16/4, FP16: 32/8, FP16 with Cin = 16: 16/4).
+// K-chunk and E elements per lane (FP32: 16/4, FP16: 32/8, FP16 with Cin = 16: 16/4, Cin = 4: 4/1).  Cin = 4
+// always takes FP32 operands (the voxel means are FP32); in an FP16 pipeline its weights are the
+// half-rounded values, as in every other layer of that pipeline.
 void pack_weights(const float* w, int K, int cin, int cout, int dtype, void* dst) {
     int C, E;
     chunk_shape(dtype, cin, &C, &E);
@@ -439,16 +443,22 @@ void pack_weights(const float* w, int K, int cin, int cout, int dtype, void* dst
                     for (int e = 0; e < E; ++e) {
                         const size_t o = ((((size_t)k * G + g) * NB + nb) * 64 + lane) * E + e;
                         const float v = w[((size_t)k * cin + C * g + E * (lane / 16) + e) * cout + 16 * nb + lane % 16];
-                        if (dtype == SESSD_HALF) static_cast<__half*>(dst)[o] = __float2half_rn(v);
+                        if (dtype == SESSD_HALF && cin != 4) static_cast<__half*>(dst)[o] = __float2half_rn(v);
+                        else if (dtype == SESSD_HALF) static_cast<float*>(dst)[o] = __half2float(__float2half_rn(v));
                         else static_cast<float*>(dst)[o] = v;
                     }
 }
 
 // -> SESSD_OK when an MFMA kernel was launched, SESSD_E_UNSUPPORTED when the shape/dtype is not covered
 int launch_mfma(const GemmArgs& a, hipStream_t stream) {
-    if (a.in_type != a.out_type || !a.w_packed || !mfma_shape(a.K, a.cin, a.cout, a.in_type)) return SESSD_E_UNSUPPORTED;
+    if (!a.w_packed || !mfma_shape(a.K, a.cin, a.cout, a.out_type)) return SESSD_E_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(a.in_feat) | reinterpret_cast<uintptr_t>(a.out_feat)) & 15)
         return SESSD_E_UNSUPPORTED;
+    if (a.cin == 4 && a.in_type == SESSD_FLOAT && a.out_type == SESSD_HALF) {  // first layer of an FP16 pipeline
+        if (a.cout == 16) return launch<float, 4, 16, __half>(a, stream);
+        if (a.cout == 32) return launch<float, 4, 32, __half>(a, stream);
+    }
+    if (a.in_type != a.out_type) return SESSD_E_UNSUPPORTED;
 #define SESSD_CASE(CI, CO)                                                        \
     if (a.cin == CI && a.cout == CO)                                              \
     return a.in_type == SESSD_HALF ? launch<__half, CI, CO>(a, stream) : launch<float, CI, CO>(a, stream)
