@@ -214,7 +214,8 @@ def main():
         ach = dom_bytes / (dom_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None}
-    kname = "conv_mfma<%s, %d, %d>" % ("__half" if args.dtype == "fp16" else "float", dom_c, dom_c)
+    tname = "__half" if args.dtype == "fp16" else "float"
+    kname = "conv_mfma<%s, %d, %d, %s>" % (tname, dom_c, dom_c, tname)
     roof["traffic"] = profiled_traffic(kname, args.dtype) if args.config == 3 else None
     roof.update({"kernel": "gather-GEMM %d->%d (%s)" % (dom_c, dom_c, args.dtype), "launches_per_frame": len(dom),
                  "avg_launch_us": round(dom_ms * 1e3, 2), "algorithmic_flops_per_launch": dom_flops,
