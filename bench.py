@@ -88,7 +88,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=3, choices=[3, 4, 5],
-                    help="BASELINE configuration: 3 = 20k points FP32 (headline), 4 = 60k points, voxel cap 40k, FP16, "
+                    help="benchmark configuration: 3 = 20k points FP32 (headline), 4 = 60k points, voxel cap 40k, FP16, "
                          "5 = 150k points over 360 degrees, voxel cap 60k, doubled channel widths, FP16")
     ap.add_argument("--points", type=int, default=None)
     ap.add_argument("--seed", type=int, default=0)

@@ -38,7 +38,7 @@ def check_voxelgen(pts, max_points, max_voxels, max_pts=5):
 
 @pytest.mark.parametrize("seed", [0, 1])
 def test_voxelgen_config2(seed):
-    """BASELINE config 2: 20 000 points, voxel 0.05x0.05x0.1, <= 5 points/voxel, cap 20 000."""
+    """Benchmark configuration 2: 20 000 points, voxel 0.05x0.05x0.1, <= 5 points/voxel, cap 20 000."""
     pts = F.lidar_frame(20000, seed)
     n = check_voxelgen(pts, 20000, 20000)
     assert 14000 < n <= 20000
@@ -108,7 +108,7 @@ def run_subm(coors_np, n, feat_np, w, grid_zyx, max_voxels, scale=None, shift=No
 
 
 def test_subm_config1_rulebook_and_features():
-    """BASELINE config 1: one SubMConv3d 4->16 on 2000 uniform voxels in 41x160x140."""
+    """Benchmark configuration 1: one SubMConv3d 4->16 on 2000 uniform voxels in 41x160x140."""
     grid = (41, 160, 140)
     n, mv = 2000, 2000
     rng = np.random.default_rng(0)
@@ -209,7 +209,7 @@ def test_mfma_and_valu_paths_agree():
 @pytest.mark.parametrize("cin,cout", [(4, 16), (16, 16), (16, 32), (32, 32), (32, 64), (64, 64), (64, 128), (128, 128),
                                       (8, 32)])
 def test_subm_fp16_features(cin, cout):
-    """FP16 features and weights, FP32 accumulate (BASELINE configs 4-5).  The oracle runs in FP32 on the
+    """FP16 features and weights, FP32 accumulate (benchmark configurations 4-5).  The oracle runs in FP32 on the
     half-rounded inputs and weights and rounds its output to half: agreement within 1e-2 relative."""
     grid = (21, 200, 176)
     n, mv = 6000, 8192

@@ -89,7 +89,7 @@ def test_pipeline_writes_the_zero_padded_dense_tensor(overlap):
 
 
 def test_full_backbone_config3_frame_and_graph_replay():
-    """BASELINE config 3: the 20 000-point frame (~17 k voxels) through the reference's 14 conv layers.
+    """Benchmark configuration 3: the 20 000-point frame (~17 k voxels) through the reference's 14 conv layers.
     The eager enqueue and repeated replays of the captured graph must give identical bits."""
     pts = F.lidar_frame(20000, 0)
     layers = B.reference_layers()
@@ -194,7 +194,7 @@ def test_properties_at_full_size():
 
 
 def test_stress_configuration_properties():
-    """BASELINE config 5: 150 000 points over 360 degrees (cropped to range), voxel cap 60 000, doubled
+    """Benchmark configuration 5: 150 000 points over 360 degrees (cropped to range), voxel cap 60 000, doubled
     channel widths, FP16 features.  Too heavy for the scalar oracle's conv layers, so: the voxelizer part
     is compared with the oracle exactly (the cap binds -> overflow flag), the rest through properties."""
     pts = F.lidar_frame(150000, 5, full_circle=True)

@@ -91,7 +91,7 @@ def test_subm_rulebook_invariants_and_brute_force(seed):
 
 
 def test_subm_rulebook_random_uniform_config1():
-    """BASELINE config 1: 2000 uniform voxels in 41x160x140."""
+    """Benchmark configuration 1: 2000 uniform voxels in 41x160x140."""
     grid = (41, 160, 140)
     coors = F.random_active_voxels(2000, grid, 0)
     pairs, num, st = O.subm_rulebook(coors, 2000, grid[::-1], 2000)
