@@ -88,6 +88,33 @@ def test_pipeline_writes_the_zero_padded_dense_tensor(overlap):
     assert np.array_equal(to_np(padded), want)
 
 
+def test_capacity_binds_in_the_voxelizer_and_in_a_strided_layer():
+    """One capacity for every tensor (as in the reference), small enough that the voxelizer drops cells and the
+    first strided layer drops output sites.  The overlapped schedule -- where SubM layers probe the cell table
+    the voxelizer / strided layer left behind, dropped cells included -- must agree with the single-stream run
+    bit for bit, and both with the oracle."""
+    pts = F.lidar_frame(6000, 13)
+    layers = B.reference_layers()
+    W = B.random_weights(layers, seed=9, w_std=0.05)
+    cap = 3000
+    ref = O.frame(pts, B.voxelgen_desc(max_voxels=cap), layers, W, B.dense_desc())
+    assert ref["status"] & D.SESSD_STATUS_VOXEL_OVERFLOW and ref["counts"][0] == cap and ref["counts"][3] == cap
+    plain, dense, _ = run_pipeline(pts, layers, W, 6000, cap, share_rulebooks=True, skip_pad_rows=True)
+    fast, fdense, (p, n, stream) = run_pipeline(pts, layers, W, 6000, cap, share_rulebooks=True, skip_pad_rows=True,
+                                                overlap_streams=True, use_graph=True)
+    with torch.cuda.stream(stream):
+        fast.enqueue(p, n, fdense, stream)                      # a replay of the captured graph
+    stream.synchronize()
+    assert np.array_equal(to_np(fdense), to_np(dense))
+    for pipe in (plain, fast):
+        assert pipe.status() == ref["status"]
+        assert [pipe.layer_count(l) for l in range(-1, len(layers))] == list(ref["counts"])
+        feat, coors, cnt = pipe.read_layer(len(layers) - 1)
+        assert np.array_equal(coors, ref["coors"])
+        assert_features_close(feat, ref["feat"], RTOL_END_TO_END, "last layer features with binding capacities")
+    assert_features_close(to_np(dense), ref["dense"], RTOL_END_TO_END, "dense tensor with binding capacities")
+
+
 def test_full_backbone_config3_frame_and_graph_replay():
     """Benchmark configuration 3: the 20 000-point frame (~17 k voxels) through the reference's 14 conv layers.
     The eager enqueue and repeated replays of the captured graph must give identical bits."""
