@@ -130,6 +130,19 @@ inline HashTable make_hash(uint32_t* keys, uint32_t* vals, uint32_t cap) {
     return t;
 }
 
+// Optional second destination of a gather-GEMM's epilogue: the dense tensor of the sparse2Dense step that
+// would follow (sparse2Dense.cu:182-207: dense[(c*D + z)][y][x] = feat[row][c], here with the zero border of
+// Sparse2DensePlugin::setPadding).  The tensor must already be cleared; its element type is the output
+// rows' type.
+struct DenseTarget {
+    void* dense = nullptr;
+    const int32_t* coors = nullptr;  // (b,z,y,x) of every output row
+    int D = 0, H = 0, W = 0;         // feature map extent the coordinates are checked against
+    int Hp = 0, Wp = 0;              // padded plane size
+    int pad_top = 0, pad_left = 0;
+    int32_t* status = nullptr;       // SESSD_STATUS_BAD_COORD is raised here
+};
+
 // ---------------------------------------------------------------------------------------------
 // fill: the only way memory is cleared (a kernel, so an enqueue can be captured in a hipGraph)
 // ---------------------------------------------------------------------------------------------

@@ -95,9 +95,15 @@ int ConvPluginBase::preparePacked() {
     return SESSD_OK;
 }
 
+bool ConvPluginBase::gemmOnMatrixCores() const {
+    return weights_packed_dev_ != nullptr && !(flags_ & SESSD_FLAG_FORCE_VALU) &&
+           gemm_runs_on_mfma(kernel_volume_, in_channel_, out_channel_, in_type_, out_type_);
+}
+
 int ConvPluginBase::runGemm(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* tiles,
-                            const int32_t* num_out, hipStream_t stream) {
+                            const int32_t* num_out, hipStream_t stream, const DenseTarget* dense) {
     GemmArgs a;
+    if (dense) a.dense = *dense;
     a.in_feat = in_feat;
     a.out_feat = out_feat;
     a.nbr = nbr;

@@ -199,6 +199,7 @@ int launch_gather_gemm(const GemmArgs& a, hipStream_t stream) {
         const int rc = launch_mfma(a, stream);
         if (rc != SESSD_E_UNSUPPORTED) return rc;  // launched (or failed for good)
     }
+    if (a.dense.dense) return fail(SESSD_E_UNSUPPORTED, "gather-GEMM: the fused dense scatter needs the MFMA kernel");
     if (!a.force_valu && a.cin == 4 && a.K <= 27 && a.in_type == SESSD_FLOAT &&
         !(reinterpret_cast<uintptr_t>(a.in_feat) & 15)) {
         // FP16 output = the FP16 configuration: half-rounded weights, as in every other layer

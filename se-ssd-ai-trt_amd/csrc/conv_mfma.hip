@@ -103,6 +103,9 @@ struct Chunk<__half, 16> {
     }
 };
 
+__device__ __forceinline__ void store1(float* dst, float v) { *dst = v; }
+__device__ __forceinline__ void store1(__half* dst, float v) { *dst = __float2half_rn(v); }
+
 // four consecutive output channels -> memory
 __device__ __forceinline__ void store4(float* dst, const float (&o)[4]) {
     *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
@@ -130,7 +133,7 @@ __global__ void __launch_bounds__(kWaves * 64, min_waves_per_simd(CIN, COUT))
 conv_mfma(const T* __restrict__ in, TO* __restrict__ out, const void* __restrict__ Wp,
           const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
           const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad,
-          int num_cu, const int32_t* __restrict__ tiles) {
+          int num_cu, const int32_t* __restrict__ tiles, DenseTarget dt) {
     using C = Chunk<T, CIN>;
     using Vec = typename C::Vec;
     constexpr int G = CIN / C::kChannels;  // K-chunks of the inner dimension
@@ -363,6 +366,17 @@ conv_mfma(const T* __restrict__ in, TO* __restrict__ out, const void* __restrict
             o[e] = s;
         }
         store4(out + (size_t)(row0 + r) * COUT + ec4, o);
+        if (dt.dense) {  // the sparse2Dense scatter of this row, fused (uniform branch)
+            const int4 cc = reinterpret_cast<const int4*>(dt.coors)[row0 + r];  // (b,z,y,x)
+            if (cc.x != 0 || cc.y < 0 || cc.y >= dt.D || cc.z < 0 || cc.z >= dt.H || cc.w < 0 || cc.w >= dt.W) {
+                if (dt.status && ec4 == 0) atomicOr(dt.status, SESSD_STATUS_BAD_COORD);
+            } else {
+                TO* d = static_cast<TO*>(dt.dense) + ((size_t)cc.y * dt.Hp + cc.z + dt.pad_top) * dt.Wp + cc.w + dt.pad_left;
+                const size_t plane = (size_t)dt.D * dt.Hp * dt.Wp;  // channel stride
+#pragma unroll
+                for (int e = 0; e < 4; ++e) store1(d + (size_t)(ec4 + e) * plane, o[e]);
+            }
+        }
     }
     __syncthreads();  // the next piece reuses the lists and partial tiles
     }
@@ -388,7 +402,8 @@ int launch(const GemmArgs& a, hipStream_t stream) {
     const unsigned blocks = (unsigned)tile_plan(a.max_voxels, num_cu).count;
     hipLaunchKernelGGL((conv_mfma<T, CIN, COUT, TO>), dim3(blocks), dim3(kWaves * 64), 0, stream,
                        static_cast<const T*>(a.in_feat), static_cast<TO*>(a.out_feat), a.w_packed, a.nbr,
-                       a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows, num_cu, a.tiles);
+                       a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows, num_cu, a.tiles,
+                       a.dense);
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;
 }
@@ -422,6 +437,11 @@ void chunk_shape(int dtype, int cin, int* channels, int* lane_elems) {
 }  // namespace
 
 int gemm_compute_units() { return compute_units(); }
+
+bool gemm_runs_on_mfma(int K, int cin, int cout, int in_type, int out_type) {
+    if (!mfma_shape(K, cin, cout, out_type)) return false;
+    return in_type == out_type || (cin == 4 && in_type == SESSD_FLOAT && out_type == SESSD_HALF);
+}
 
 size_t packed_weight_bytes(int K, int cin, int cout, int dtype) {
     if (!mfma_shape(K, cin, cout, dtype)) return 0;

@@ -22,6 +22,7 @@ struct GemmArgs {
     int write_pad_rows;      // rows >= *num_out get epilogue(0) (the reference zero-fills them)
     int force_valu;          // skip the MFMA kernels (cross-check)
     const int32_t* tiles;    // tile cuts of this rulebook (launch_tile_cuts) or null: tiles of equal length
+    DenseTarget dense;       // dense.dense != null: also scatter the rows there (MFMA kernel only)
 };
 
 // Tiling of the MFMA gather-GEMM: n active rows on num_cu compute units are cut into num_cu * r tiles,
@@ -57,8 +58,10 @@ size_t tile_cut_bytes(int max_voxels);
 int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, void* region,
                      hipStream_t stream);
 
-// picks the kernel for the layer shape; returns SESSD_E_UNSUPPORTED for dtype pairs not covered
+// picks the kernel for the layer shape; returns SESSD_E_UNSUPPORTED for dtype pairs not covered, and when a
+// dense target is set but the layer does not run on the MFMA kernel (see gemm_runs_on_mfma)
 int launch_gather_gemm(const GemmArgs& a, hipStream_t stream);
+bool gemm_runs_on_mfma(int K, int cin, int cout, int in_type, int out_type);
 
 // size in bytes of the packed weight copy for this shape/dtype (0 = shape runs on the VALU path)
 size_t packed_weight_bytes(int K, int cin, int cout, int dtype);

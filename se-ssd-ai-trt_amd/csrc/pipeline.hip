@@ -158,6 +158,7 @@ struct Pipeline {
         coors = static_cast<const int32_t*>(vg_coors.p);
         num = static_cast<const int32_t*>(vg_num.p);
         int last_waited = -1;
+        bool scattered = false;
         for (size_t l = 0; l < stages.size(); ++l) {
             ConvStage& st = *stages[l];
             const int owner = st.rulebook_from >= 0 ? st.rulebook_from : (int)l;
@@ -165,15 +166,30 @@ struct Pipeline {
                 SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_build[owner], 0));
                 last_waited = owner;
             }
+            // the last layer's epilogue also writes the dense tensor when it runs on the matrix cores and its
+            // rows have the dense tensor's element type: the scatter kernel and its launch drop off the end
+            // of the critical path
+            ConvPluginBase* cp = st.subm ? static_cast<ConvPluginBase*>(st.subm.get()) : st.sparse.get();
+            DenseTarget dt;
+            const bool fuse = l + 1 == stages.size() && cp->out_type_ == s2d->out_type_ &&
+                              cp->out_channel_ == s2d->feature_map_channel_ && cp->gemmOnMatrixCores();
+            if (fuse) {
+                SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_fill, 0));
+                const int32_t* oc = st.subm ? coors : static_cast<const int32_t*>(st.coors.p);
+                dt = s2d->denseTarget(dense, oc, s2d_ws.p);
+                scattered = true;
+            }
             if (st.subm) {
-                SESSD_TRY(st.subm->enqueueGemm(feat, st.feat.p, num, stages[owner]->ws.p, stream));
+                SESSD_TRY(st.subm->enqueueGemm(feat, st.feat.p, num, stages[owner]->ws.p, stream, fuse ? &dt : nullptr));
             } else {
-                SESSD_TRY(st.sparse->enqueueGemm(feat, st.feat.p, static_cast<const int32_t*>(st.num.p), st.ws.p, stream));
+                SESSD_TRY(st.sparse->enqueueGemm(feat, st.feat.p, static_cast<const int32_t*>(st.num.p), st.ws.p, stream,
+                                                 fuse ? &dt : nullptr));
                 coors = static_cast<const int32_t*>(st.coors.p);
                 num = static_cast<const int32_t*>(st.num.p);
             }
             feat = st.feat.p;
         }
+        if (scattered) return SESSD_OK;
         // every event of `aux` has been waited on by now (the last build is the last aux operation)
         if (stages.empty()) SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_vg, 0));
         SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_fill, 0));

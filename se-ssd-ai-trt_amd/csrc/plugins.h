@@ -71,6 +71,8 @@ class ConvPluginBase {
     int uploadWeights(const float* w, size_t count);
     int configureTypes(const sessd_tensor_desc* in, int nbInputs, const sessd_tensor_desc* out,
                        int nbOutputs);
+    // whether this layer's gather-GEMM runs on the MFMA kernel (the one that can take a DenseTarget)
+    bool gemmOnMatrixCores() const;
 
     int in_channel_ = 0, out_channel_ = 0, max_voxels_ = 0, feature_num_ = 0;
     int out_shape_x_ = 0, out_shape_y_ = 0, out_shape_z_ = 0;
@@ -91,8 +93,9 @@ class ConvPluginBase {
 
   protected:
     // gather-GEMM over the neighbour table nbr[K][max_voxels] (device), rows < *num_out
+    // `dense`: also scatter the output rows into the dense tensor of a sparse2Dense step (MFMA kernel only)
     int runGemm(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* tiles,
-                const int32_t* num_out, hipStream_t stream);
+                const int32_t* num_out, hipStream_t stream, const DenseTarget* dense = nullptr);
     // whether a rulebook built by this layer gets equal-work tile cuts: worth two small launches when the
     // GEMM runs on the matrix cores and is not tiny
     bool wantTileCuts() const {
@@ -131,7 +134,7 @@ class SubmConv3dLayerPlugin : public ConvPluginBase {
                      bool prefilled = false, const HashTable* cells = nullptr);
     void collectFill(void* workspace, FillArgs& f) const;
     int enqueueGemm(const void* in_feat, void* out_feat, const int32_t* voxel_num,
-                    const void* rulebook_workspace, hipStream_t stream);
+                    const void* rulebook_workspace, hipStream_t stream, const DenseTarget* dense = nullptr);
     int exportRulebook(const void* workspace, int32_t* indice_pairs, uint32_t* indice_num,
                        hipStream_t stream) const;
     int countPairs(const void* workspace, uint32_t* indice_num, hipStream_t stream) const;
@@ -172,7 +175,7 @@ class SparseConv3dLayerPlugin : public ConvPluginBase {
     HashTable cellTable(void* workspace) const;
     void collectFill(void* workspace, int32_t* out_coors, FillArgs& f) const;
     int enqueueGemm(const void* in_feat, void* out_feat, const int32_t* out_num, const void* workspace,
-                    hipStream_t stream);
+                    hipStream_t stream, const DenseTarget* dense = nullptr);
     size_t getSerializationSize() const;
     void serialize(void* buffer) const;
     size_t statusOffset() const;
@@ -203,6 +206,8 @@ class Sparse2DensePlugin {
                 const void* const* inputs, void* const* outputs, void* workspace,
                 hipStream_t stream, bool prefilled = false);
     void collectFill(void* dense, void* workspace, FillArgs& f) const;
+    // the scatter of enqueue() as an epilogue of the gather-GEMM that produces `coors`' feature rows
+    DenseTarget denseTarget(void* dense, const int32_t* coors, void* workspace) const;
     size_t getSerializationSize() const;
     void serialize(void* buffer) const;
 

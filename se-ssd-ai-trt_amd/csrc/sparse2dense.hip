@@ -142,6 +142,21 @@ void Sparse2DensePlugin::collectFill(void* dense, void* workspace, FillArgs& f) 
     if (workspace) f.add(workspace, 4, 0);
 }
 
+DenseTarget Sparse2DensePlugin::denseTarget(void* dense, const int32_t* coors, void* workspace) const {
+    DenseTarget t;
+    t.dense = dense;
+    t.coors = coors;
+    t.D = feature_map_size_z_;
+    t.H = feature_map_size_y_;
+    t.W = feature_map_size_x_;
+    t.Hp = outHeight();
+    t.Wp = outWidth();
+    t.pad_top = zero_padding_2d_top_;
+    t.pad_left = zero_padding_2d_left_;
+    t.status = static_cast<int32_t*>(workspace);
+    return t;
+}
+
 int Sparse2DensePlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
                                 const void* const* inputs, void* const* outputs, void* workspace,
                                 hipStream_t stream, bool prefilled) {

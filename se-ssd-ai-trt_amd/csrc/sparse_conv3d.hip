@@ -392,10 +392,10 @@ HashTable SparseConv3dLayerPlugin::cellTable(void* workspace) const {
 }
 
 int SparseConv3dLayerPlugin::enqueueGemm(const void* in_feat, void* out_feat, const int32_t* out_num,
-                                         const void* workspace, hipStream_t stream) {
+                                         const void* workspace, hipStream_t stream, const DenseTarget* dense) {
     if (!in_feat || !out_feat || !out_num || !workspace) return fail(SESSD_E_INVALID, "sparseconv3d.gemm: null pointer");
     const Layout L = carve(const_cast<void*>(workspace));
-    return runGemm(in_feat, out_feat, L.nbr, L.tiles, out_num, stream);
+    return runGemm(in_feat, out_feat, L.nbr, L.tiles, out_num, stream, dense);
 }
 
 int SparseConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,

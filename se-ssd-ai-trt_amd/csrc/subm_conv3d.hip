@@ -257,11 +257,12 @@ int SubmConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* vox
 }
 
 int SubmConv3dLayerPlugin::enqueueGemm(const void* in_feat, void* out_feat, const int32_t* voxel_num,
-                                       const void* rulebook_workspace, hipStream_t stream) {
+                                       const void* rulebook_workspace, hipStream_t stream,
+                                       const DenseTarget* dense) {
     if (!in_feat || !out_feat || !voxel_num || !rulebook_workspace)
         return fail(SESSD_E_INVALID, "submconv3d.gemm: null pointer");
     const Layout L = carve(const_cast<void*>(rulebook_workspace));
-    return runGemm(in_feat, out_feat, L.nbr, L.tiles, voxel_num, stream);
+    return runGemm(in_feat, out_feat, L.nbr, L.tiles, voxel_num, stream, dense);
 }
 
 int SubmConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
