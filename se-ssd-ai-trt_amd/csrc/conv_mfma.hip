@@ -311,7 +311,13 @@ conv_mfma(const T* __restrict__ in, TO* __restrict__ out, const void* __restrict
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) C::mma(b[g][nb], a_cur[blk][g], acc[blk][nb]);
             }
-            if (k_nxt >= 0) load_b(k_nxt, g, b[g]);
+            // The next offset's chunk g replaces this one.  FP16: requested unconditionally (after the last
+            // offset the same chunk once more), because a load under a branch makes the compiler's count of
+            // loads in flight inexact and every later wait a wait for nearly all of them, the rows just
+            // requested included.  FP32 chunks are twice the bytes and their MFMAs four times as long: there
+            // the redundant last request costs more than the exact waits save (measured).
+            if constexpr (sizeof(T) == 2) load_b(k_nxt >= 0 ? k_nxt : k_cur, g, b[g]);
+            else if (k_nxt >= 0) load_b(k_nxt, g, b[g]);
         }
         // block results -> partial tile.  D is the transposed block: lane (pair j = lane%16, q = lane/16)
         // holds output channels 16nb+4q .. +3 of pair j -- one 16-byte LDS read-modify-write per column
