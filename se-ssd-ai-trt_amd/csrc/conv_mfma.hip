@@ -10,9 +10,9 @@
 //     with wave64 ballot + popcount: pair list k = the (input row, local output row) pairs of the rows
 //     that really have a neighbour at offset k.  Only those rows enter an MFMA block, so the matrix
 //     cores do not multiply the zero rows a dense [rows x K*Cin] gather matrix would be half full of.
-//   * Non-empty offsets are dealt to the four waves, longest pair list first, each to the wave with the
-//     least work so far (split-K over offsets): tiles x 4 waves is what fills 256 CUs with a ~17k-row
-//     problem.
+//   * Non-empty offsets are dealt to the four waves (split-K over offsets), ranked by their number of
+//     16-pair blocks and dealt back and forth (0 1 2 3 3 2 1 0 ...): tiles x 4 waves is what fills 256 CUs
+//     with a ~17k-row problem.
 //   * A wave gathers 16 pairs per MFMA block straight into operand registers: lane (i = lane%16,
 //     q = lane/16) loads 16 bytes of pair i's input row per K-chunk (FP32: channels 16g+4q..+3, FP16:
 //     channels 32g+8q..+7), i.e. every row is read as 64-byte segments.  The weights were reordered on
@@ -28,6 +28,8 @@
 //     measured several times slower).
 //   * The four partial tiles are summed in a fixed order, scale/shift/ReLU is applied in FP32 and each
 //     output row is written once, coalesced.  No global atomics; results are bit-identical run to run.
+//     A caller may name a dense tensor (DenseTarget): the epilogue then also stores every row at its voxel's
+//     place there, which is the sparse2Dense step that follows the last layer.
 #include "kernels.h"
 
 namespace sessd {
