@@ -97,6 +97,12 @@ struct Pipeline {
     int enqueueOverlapped(const void* points, const void* points_size, void* dense, hipStream_t stream) {
         SESSD_HIP_TRY(hipEventRecord(ev_start, stream));
         SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_start, 0));
+        // The voxelizer heads the frame's critical path: it is queued (and, in a graph, submitted) before
+        // anything else.
+        const void* vin[2] = {points, points_size};
+        void* vout[3] = {vg_voxels.p, vg_coors.p, vg_num.p};
+        SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, aux));
+        SESSD_HIP_TRY(hipEventRecord(ev_vg, aux));
         SESSD_HIP_TRY(hipStreamWaitEvent(aux_fill, ev_start, 0));
         // every clear of the frame (hash tables, neighbour tables, status words, the dense tensor) has no
         // input: they run batched on a third stream while the voxelizer works
@@ -118,10 +124,6 @@ struct Pipeline {
             SESSD_TRY(flush());
             SESSD_HIP_TRY(hipEventRecord(ev_fill, aux_fill));
         }
-        const void* vin[2] = {points, points_size};
-        void* vout[3] = {vg_voxels.p, vg_coors.p, vg_num.p};
-        SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, aux));
-        SESSD_HIP_TRY(hipEventRecord(ev_vg, aux));
         SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_fill, 0));
         const int32_t* coors = static_cast<const int32_t*>(vg_coors.p);
         const int32_t* num = static_cast<const int32_t*>(vg_num.p);
