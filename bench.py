@@ -46,6 +46,18 @@ def profiled_traffic(kernel, dtype):
     return None
 
 
+def cpu_model():
+    """Model name of the host CPU as /proc/cpuinfo gives it."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown CPU"
+
+
 def cpu_baseline(pts, layers, W, max_voxels, voxel_cap, budget_s=24.0):
     """The CPU port (the parity oracle) on the same frame, a bounded number of frames: once on one thread and
     once with the pairs of every kernel offset split over the host's cores (same bits either way)."""
@@ -79,7 +91,8 @@ def cpu_baseline(pts, layers, W, max_voxels, voxel_cap, budget_s=24.0):
             "single_thread_ms": round(one, 2),
             "sample": "the same %d-point frame through oracle_frame (g++ -O2): median of %d frame(s) with the gather-GEMM's "
                       "pairs split over %d threads (value), median of %d frame(s) on one thread (single_thread_ms); "
-                      "host reports %d logical CPUs" % (len(pts), n_many, threads, n_one, os.cpu_count() or 0)}
+                      "host reports %d logical CPUs (%s)" % (len(pts), n_many, threads, n_one, os.cpu_count() or 0,
+                                                               cpu_model())}
 
 
 def main():
