@@ -115,6 +115,36 @@ def test_capacity_binds_in_the_voxelizer_and_in_a_strided_layer():
     assert_features_close(to_np(dense), ref["dense"], RTOL_END_TO_END, "dense tensor with binding capacities")
 
 
+def test_overlapped_graph_schedule_with_reference_pad_rows():
+    """Reference behaviour for rows past the active count (every output tensor is zero-filled, then BN + ReLU
+    runs over all rows: rows >= n hold relu(shift)) under the overlapped schedule and its captured graph: dense
+    tensor, active rows and pad rows must equal the single-stream run bit for bit, frame after frame."""
+    pts = F.lidar_frame(3000, 17)
+    layers = B.reference_layers()
+    W = B.random_weights(layers, seed=12, w_std=0.05)
+    mv = 8192
+    plain, dense, _ = run_pipeline(pts, layers, W, 4096, mv, share_rulebooks=True, skip_pad_rows=False)
+    fast, fdense, (p, n, stream) = run_pipeline(pts, layers, W, 4096, mv, share_rulebooks=True, skip_pad_rows=False,
+                                                overlap_streams=True, use_graph=True)
+    for _ in range(2):                                               # graph replays
+        with torch.cuda.stream(stream):
+            fast.enqueue(p, n, fdense, stream)
+        stream.synchronize()
+        assert np.array_equal(to_np(fdense), to_np(dense))
+    assert fast.status() == plain.status() == 0
+    for l in (0, 5, len(layers) - 1):
+        rows = []
+        for pipe in (plain, fast):
+            f, _, _, _, ch = pipe.layer_io(l)
+            full = np.zeros((mv, ch), np.float32)
+            api._hip_d2h(full, f)
+            rows.append((full, 0))
+        assert np.array_equal(rows[0][0], rows[1][0]), layers[l].name
+        cnt = plain.layer_count(l)
+        want_pad = np.maximum(W.shift[l], 0.0).astype(np.float32)    # relu(0 * scale + shift)
+        assert np.array_equal(rows[0][0][cnt:], np.broadcast_to(want_pad, (mv - cnt, len(want_pad)))), layers[l].name
+
+
 def test_full_backbone_config3_frame_and_graph_replay():
     """Benchmark configuration 3: the 20 000-point frame (~17 k voxels) through the reference's 14 conv layers.
     The eager enqueue and repeated replays of the captured graph must give identical bits."""
