@@ -103,6 +103,29 @@ struct Pipeline {
         void* vout[3] = {vg_voxels.p, vg_coors.p, vg_num.p};
         SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, aux));
         SESSD_HIP_TRY(hipEventRecord(ev_vg, aux));
+        // The kernel that produced a coors tensor has left a cell -> row hash behind (the voxelizer's, or a
+        // strided layer's): a SubM layer on the same grid looks its neighbours up in that table and skips its
+        // own insert pass (and the clear of its own table).  Keys are (z*Y + y)*X + x: the same number in both
+        // grids when X and Y agree; cells of the layer's grid beyond the table's z extent are simply absent.
+        // (Beyond 2^20 slots -- 4 MB of keys, one XCD's L2 -- probing the upstream table costs more than the
+        // insert pass it saves.)
+        std::vector<char> probes_upstream(stages.size(), 0);
+        {
+            uint32_t mask = vg->cellTable(vg_ws.p, desc.max_points).mask;
+            int cx = vg->grid_x_size_, cy = vg->grid_y_size_, cz = vg->grid_z_size_;
+            for (size_t l = 0; l < stages.size(); ++l) {
+                ConvStage& st = *stages[l];
+                if (st.subm) {
+                    probes_upstream[l] = st.rulebook_from < 0 && st.subm->out_shape_x_ == cx &&
+                                         st.subm->out_shape_y_ == cy && st.subm->out_shape_z_ >= cz && mask < (1u << 20);
+                } else {
+                    mask = st.sparse->cellTable(st.ws.p).mask;
+                    cx = st.sparse->out_shape_x_;
+                    cy = st.sparse->out_shape_y_;
+                    cz = st.sparse->out_shape_z_;
+                }
+            }
+        }
         SESSD_HIP_TRY(hipStreamWaitEvent(aux_fill, ev_start, 0));
         // every clear of the frame (hash tables, neighbour tables, status words, the dense tensor) has no
         // input: they run batched on a third stream while the voxelizer works
@@ -113,10 +136,11 @@ struct Pipeline {
                 f = FillArgs();
                 return rc;
             };
-            for (auto& st : stages) {
+            for (size_t l = 0; l < stages.size(); ++l) {
+                auto& st = stages[l];
                 if (!st->ws.p) continue;
                 if (f.n + 5 > FillArgs::kMaxRegions) SESSD_TRY(flush());
-                if (st->subm) st->subm->collectFill(st->ws.p, f);
+                if (st->subm) st->subm->collectFill(st->ws.p, f, !probes_upstream[l]);
                 else st->sparse->collectFill(st->ws.p, static_cast<int32_t*>(st->coors.p), f);
             }
             if (f.n + 2 > FillArgs::kMaxRegions) SESSD_TRY(flush());
@@ -127,31 +151,18 @@ struct Pipeline {
         SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_fill, 0));
         const int32_t* coors = static_cast<const int32_t*>(vg_coors.p);
         const int32_t* num = static_cast<const int32_t*>(vg_num.p);
-        // The kernel that produced a coors tensor has left a cell -> row hash behind (the voxelizer's, or a
-        // strided layer's): a SubM layer on the same grid looks its neighbours up in that table and skips its
-        // own insert pass.  `cells` = that table, {cx, cy, cz} = the x/y grid it is keyed on and its z extent.
-        HashTable cells = vg->cellTable(vg_ws.p, desc.max_points);
-        int cx = vg->grid_x_size_, cy = vg->grid_y_size_, cz = vg->grid_z_size_;
+        HashTable cells = vg->cellTable(vg_ws.p, desc.max_points);  // the table upstream of the current layer
         for (size_t l = 0; l < stages.size(); ++l) {
             ConvStage& st = *stages[l];
             if (st.subm) {
                 if (st.rulebook_from >= 0) continue;
-                // keys are (z*Y + y)*X + x: the same number in both grids when X and Y agree; cells of the
-                // layer's grid beyond the table's z extent are simply absent
-                // (a strided layer's table is sized for every candidate cell of max_voxels inputs; beyond 2^20
-                // slots -- 4 MB of keys, one XCD's L2 -- probing it costs more than the insert pass it saves)
-                const bool same_grid = st.subm->out_shape_x_ == cx && st.subm->out_shape_y_ == cy &&
-                                       st.subm->out_shape_z_ >= cz && cells.mask < (1u << 20);
-                SESSD_TRY(st.subm->enqueueBuild(coors, num, st.ws.p, aux, true, same_grid ? &cells : nullptr));
+                SESSD_TRY(st.subm->enqueueBuild(coors, num, st.ws.p, aux, true, probes_upstream[l] ? &cells : nullptr));
             } else {
                 SESSD_TRY(st.sparse->enqueueBuild(coors, num, static_cast<int32_t*>(st.coors.p),
                                                   static_cast<int32_t*>(st.num.p), st.ws.p, aux, true));
                 coors = static_cast<const int32_t*>(st.coors.p);
                 num = static_cast<const int32_t*>(st.num.p);
                 cells = st.sparse->cellTable(st.ws.p);
-                cx = st.sparse->out_shape_x_;
-                cy = st.sparse->out_shape_y_;
-                cz = st.sparse->out_shape_z_;
             }
             SESSD_HIP_TRY(hipEventRecord(ev_build[l], aux));
         }

@@ -132,7 +132,7 @@ class SubmConv3dLayerPlugin : public ConvPluginBase {
     // voxelizer's, or that of the strided layer that produced `coors`); the insert pass is skipped then
     int enqueueBuild(const int32_t* coors, const int32_t* voxel_num, void* workspace, hipStream_t stream,
                      bool prefilled = false, const HashTable* cells = nullptr);
-    void collectFill(void* workspace, FillArgs& f) const;
+    void collectFill(void* workspace, FillArgs& f, bool own_table = true) const;
     int enqueueGemm(const void* in_feat, void* out_feat, const int32_t* voxel_num,
                     const void* rulebook_workspace, hipStream_t stream, const DenseTarget* dense = nullptr);
     int exportRulebook(const void* workspace, int32_t* indice_pairs, uint32_t* indice_num,

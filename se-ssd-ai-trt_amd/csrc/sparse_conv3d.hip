@@ -110,7 +110,7 @@ sp_flags(const int32_t* __restrict__ voxel_num, SpParams P, HashTable t, const u
 __global__ void __launch_bounds__(kBlock)
 sp_number(SpParams P, HashTable t, const uint32_t* __restrict__ cand, const uint64_t* __restrict__ first_words,
           const uint32_t* __restrict__ block_counts, int n_blocks, int32_t* __restrict__ out_coors,
-          int32_t* __restrict__ out_num, int32_t* meta) {
+          int32_t* __restrict__ out_num, int32_t* __restrict__ nbr, int K, int32_t* meta) {
     __shared__ uint32_t lds4[4];
     const int b = blockIdx.x;
     const int upto = b == 0 ? n_blocks : b;  // block 0 computes the total
@@ -145,6 +145,9 @@ sp_number(SpParams P, HashTable t, const uint32_t* __restrict__ cand, const uint
     const int rem = key - z * plane;
     const int y = rem / P.os[2];
     reinterpret_cast<int4*>(out_coors)[id] = make_int4(0, z, y, rem - y * P.os[2]);  // sparseConv3dlayer.cu:438-441
+    // the new row's neighbour entries start empty (sp_scatter fills in the pairs): clearing them here, row by
+    // row, instead of the whole K x max_voxels table before the frame touches only the rows that exist
+    for (int k = 0; k < K; ++k) nbr[(size_t)k * P.max_voxels + id] = -1;
 }
 
 __global__ void __launch_bounds__(kBlock)
@@ -353,7 +356,6 @@ size_t SparseConv3dLayerPlugin::statusOffset() const { return carve(nullptr).met
 void SparseConv3dLayerPlugin::collectFill(void* workspace, int32_t* out_coors, FillArgs& f) const {
     const Layout L = carve(workspace);
     f.add(L.keys, (uint64_t)L.cap * 2, kEmpty);
-    f.add(L.nbr, (uint64_t)kernel_volume_ * max_voxels_, kEmpty);  // -1 = no input at this offset
     f.add(L.tiles, 4, 0);
     f.add(L.meta, 4, 0);
     if (!(flags_ & SESSD_FLAG_SKIP_PAD_ROWS)) f.add(out_coors, (uint64_t)max_voxels_ * 4, 0);  // :668
@@ -385,7 +387,7 @@ int SparseConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* v
     hipLaunchKernelGGL(sp_insert, grid, block, 0, stream, coors, voxel_num, P, t, L.cand, L.meta);
     hipLaunchKernelGGL(sp_flags, grid, block, 0, stream, voxel_num, P, t, L.cand, L.first_words, L.block_counts);
     hipLaunchKernelGGL(sp_number, grid, block, 0, stream, P, t, L.cand, L.first_words, L.block_counts,
-                       L.n_blocks, out_coors, out_num, L.meta);
+                       L.n_blocks, out_coors, out_num, L.nbr, kernel_volume_, L.meta);
     hipLaunchKernelGGL(sp_scatter, grid, block, 0, stream, voxel_num, P, t, L.cand, L.nbr);
     SESSD_HIP_TRY(hipGetLastError());
     if (wantTileCuts()) SESSD_TRY(launch_tile_cuts(L.nbr, out_num, kernel_volume_, max_voxels_, L.tiles, stream));

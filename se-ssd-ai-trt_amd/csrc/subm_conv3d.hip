@@ -226,9 +226,9 @@ size_t SubmConv3dLayerPlugin::statusOffset() const { return carve(nullptr).meta_
 // rulebook and the features: a pipeline may run the halves of different layers on different streams.
 // what enqueueBuild clears before it launches anything: a caller that batches the clears of many layers
 // into one launch collects them with this and passes prefilled = true
-void SubmConv3dLayerPlugin::collectFill(void* workspace, FillArgs& f) const {
+void SubmConv3dLayerPlugin::collectFill(void* workspace, FillArgs& f, bool own_table) const {
     const Layout L = carve(workspace);
-    f.add(L.keys, (uint64_t)L.cap * 2, kEmpty);
+    if (own_table) f.add(L.keys, (uint64_t)L.cap * 2, kEmpty);  // (not when the build probes another table)
     f.add(L.tiles, 4, 0);
     f.add(L.meta, 4, 0);
 }
