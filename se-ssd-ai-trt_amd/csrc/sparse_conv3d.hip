@@ -183,6 +183,12 @@ struct SparseConv3dLayerPlugin::Layout {
     size_t total;
 };
 
+// slots of the candidate hash beyond the worst-case number of distinct candidates: 1/kHashSlack of it
+#ifndef SESSD_SP_HASH_SLACK
+#define SESSD_SP_HASH_SLACK 16
+#endif
+constexpr uint64_t kHashSlack = SESSD_SP_HASH_SLACK;
+
 int SparseConv3dLayerPlugin::maxCandidates() const {
     const int k[3] = {ksize0_, ksize1_, ksize2_}, s[3] = {stride0_, stride1_, stride2_};
     int kc = 1;
@@ -198,13 +204,10 @@ SparseConv3dLayerPlugin::Layout SparseConv3dLayerPlugin::carve(void* workspace) 
     uint64_t distinct = (uint64_t)L.Kc * max_voxels_;  // upper bound on distinct candidate cells
     if (distinct > volume) distinct = volume;
     if (distinct < 32) distinct = 32;
-#ifndef SESSD_SP_HASH_SLACK
-#define SESSD_SP_HASH_SLACK 16
-#endif
     // every distinct candidate cell gets a slot (the cap on output rows applies after numbering).  The bound is
     // the worst case -- every input row with Kc candidates of its own -- of which a real frame uses a few per
     // cent, so the table is sized just above it rather than at twice it: half the bytes to clear per frame.
-    L.cap = next_pow2(distinct + distinct / SESSD_SP_HASH_SLACK);
+    L.cap = next_pow2(distinct + distinct / kHashSlack);
     const int64_t tickets = (int64_t)L.Kc * max_voxels_;
     L.n_blocks = ceil_div(tickets, kBlock);
     L.keys = c.take<uint32_t>((size_t)L.cap * 2);
