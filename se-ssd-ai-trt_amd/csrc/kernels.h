@@ -29,8 +29,10 @@ struct GemmArgs {
 // r = the smallest tiles-per-CU count that keeps the mean tile at or below the target height, so that every
 // CU gets the same number of tiles (a fixed 32-row tiling leaves e.g. 529 tiles for 256 CUs: some CUs run
 // three tiles, most two, and the kernel lasts as long as the three).
+// The target is the kernel's tile capacity: the tallest tiles the quantisation to whole tiles per CU allows
+// (runs the equal-work cuts make longer than the capacity are walked in pieces by the kernel).
 #ifndef SESSD_GEMM_TARGET_ROWS
-#define SESSD_GEMM_TARGET_ROWS 40
+#define SESSD_GEMM_TARGET_ROWS 48
 #endif
 constexpr int kGemmTargetRows = SESSD_GEMM_TARGET_ROWS;
 constexpr int kGemmMaxOffsets = 27;  // kernel volumes the rulebook holds (3 x 3 x 3)
