@@ -296,6 +296,11 @@ conv_mfma(const T* __restrict__ in, TO* __restrict__ out, const void* __restrict
     while (k_cur >= 0) {
         const int k_nxt = my_mask ? __ffs(my_mask) - 1 : -1;
         my_mask &= my_mask - 1;
+        // Everything requested during the previous offset is consumed by this one: wait for all of it here,
+        // before this offset's own requests go out.  Left to itself the compiler waits chunk by chunk, and
+        // because some requests sit under branches its count is inexact: the wait before the second chunk then
+        // also covers the rows and weights requested a moment ago for the NEXT offset.
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         if (k_nxt >= 0) {
             cnt_nxt = __builtin_amdgcn_readfirstlane(s_cnt[k_nxt]);  // wave-uniform: keep it scalar
             load_a(k_nxt, cnt_nxt, a_nxt);
