@@ -46,12 +46,20 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 #ifndef SESSD_MFMA_TM
 #define SESSD_MFMA_TM 48
 #endif
+#ifndef SESSD_MFMA_TM_WIDE_F16
+#define SESSD_MFMA_TM_WIDE_F16 64
+#endif
 constexpr int kWaves = SESSD_MFMA_WAVES;
-constexpr int kTileRows = SESSD_MFMA_TM;        // capacity: most output rows a workgroup can own (<= 64)
-constexpr int kMaxBlk = (kTileRows + 15) / 16;  // MFMA row blocks an offset can need
 constexpr int kMaxK = kGemmMaxOffsets;
 
-static_assert(kGemmTargetRows <= kTileRows && kTileRows <= 64, "tile height must fit the capacity and one wave");
+// Tile capacity: most output rows a workgroup can own (<= 64: one wave stages a neighbour list).  The rows
+// of all blocks of two offsets live in registers, so the capacity is what the register file allows: 48 rows
+// for FP32 (64 spill in the 64-wide layers), 64 for the wide FP16 layers, whose rows take half the registers
+// and whose launches are short enough for one tile per CU less to show.  The narrow FP16 layers and
+// Cin = 128 measured slower with 64.
+constexpr int tile_rows(bool half_operands, int cin, int cout) {
+    return half_operands && cin <= 64 && cin * cout >= 32 * 64 ? SESSD_MFMA_TM_WIDE_F16 : SESSD_MFMA_TM;
+}
 
 // Per-dtype shape of one K-chunk: how many channels it spans, what a lane holds of it, and the MFMA
 // sequence that consumes it (w = weights fragment -> A operand, x = gathered-row fragment -> B operand).
@@ -150,13 +158,16 @@ conv_mfma(const T* __restrict__ in, TO* __restrict__ out, const void* __restrict
     constexpr int CW = COUT / CS;            // columns of one wave
     constexpr int LDP = CW + 4;              // padded row stride of the partial tiles in LDS
     static_assert(CIN % C::kChannels == 0 && COUT % 16 == 0, "channel counts must fill whole MFMA chunks");
+    constexpr int kTileRows = tile_rows(sizeof(T) == 2, CIN, COUT);
+    constexpr int kMaxBlk = (kTileRows + 15) / 16;  // MFMA row blocks an offset can need
+    static_assert(kGemmMinTileRows <= kTileRows && kTileRows <= 64, "capacity: at least the bound the grid is sized with, at most one wave");
     __shared__ int32_t s_in[kMaxK * kTileRows];   // compacted pair lists: input row ...
     __shared__ uint8_t s_row[kMaxK * kTileRows];  // ... and local output row of pair j of offset k
     __shared__ int32_t s_cnt[kMaxK + 5];          // pairs per offset
     __shared__ float s_part[kWaves * kTileRows * LDP];
 
-    // the row count and the tile cuts are independent loads: request them together (a grid of
-    // tile_plan(max_voxels).count workgroups never indexes past the cut table)
+    // the row count and the tile cuts are independent loads: request them together (the grid is sized for
+    // the smallest tile height any rulebook is cut for and never indexes past the cut table)
     int n = *num_out;
     const int cut_count = tiles ? tiles[0] : 0;
     const int cut_begin = tiles ? tiles[4 + blockIdx.x] : 0;
@@ -203,7 +214,7 @@ conv_mfma(const T* __restrict__ in, TO* __restrict__ out, const void* __restrict
         run_begin = cut_begin;
         run_end = cut_end;
     } else {
-        const int R = tile_plan(n, num_cu).height;
+        const int R = tile_plan(n, num_cu, kTileRows).height;
         run_begin = blockIdx.x * R;
         run_end = run_begin + R < n ? run_begin + R : n;
     }
@@ -411,8 +422,9 @@ int compute_units() {
 template <typename T, int CIN, int COUT, typename TO = T>
 int launch(const GemmArgs& a, hipStream_t stream) {
     const int num_cu = compute_units();
-    // tile_plan() never cuts n <= max_voxels rows into more tiles than it does max_voxels rows
-    const unsigned blocks = (unsigned)tile_plan(a.max_voxels, num_cu).count;
+    // enough workgroups for any cut of any n <= max_voxels rows: tile_plan() never makes more tiles for fewer
+    // rows or a taller target (surplus workgroups return at once)
+    const unsigned blocks = (unsigned)tile_plan(a.max_voxels, num_cu, kGemmMinTileRows).count;
     hipLaunchKernelGGL((conv_mfma<T, CIN, COUT, TO>), dim3(blocks), dim3(kWaves * 64), 0, stream,
                        static_cast<const T*>(a.in_feat), static_cast<TO*>(a.out_feat), a.w_packed, a.nbr,
                        a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows, num_cu, a.tiles,
@@ -450,6 +462,8 @@ void chunk_shape(int dtype, int cin, int* channels, int* lane_elems) {
 }  // namespace
 
 int gemm_compute_units() { return compute_units(); }
+
+int gemm_tile_rows(int cin, int cout, int dtype) { return tile_rows(dtype == SESSD_HALF && cin != 4, cin, cout); }
 
 bool gemm_runs_on_mfma(int K, int cin, int cout, int in_type, int out_type) {
     if (!mfma_shape(K, cin, cout, out_type)) return false;

@@ -29,36 +29,40 @@ struct GemmArgs {
 // r = the smallest tiles-per-CU count that keeps the mean tile at or below the target height, so that every
 // CU gets the same number of tiles (a fixed 32-row tiling leaves e.g. 529 tiles for 256 CUs: some CUs run
 // three tiles, most two, and the kernel lasts as long as the three).
-// The target is the kernel's tile capacity: the tallest tiles the quantisation to whole tiles per CU allows
-// (runs the equal-work cuts make longer than the capacity are walked in pieces by the kernel).
-#ifndef SESSD_GEMM_TARGET_ROWS
-#define SESSD_GEMM_TARGET_ROWS 48
+// The target is the tile capacity of the kernel the rulebook's owner runs (gemm_tile_rows()): the tallest
+// tiles the quantisation to whole tiles per CU allows.  Any cut is correct for any kernel: runs longer than
+// a kernel's capacity are walked in pieces.
+#ifndef SESSD_GEMM_MIN_TILE_ROWS
+#define SESSD_GEMM_MIN_TILE_ROWS 48
 #endif
-constexpr int kGemmTargetRows = SESSD_GEMM_TARGET_ROWS;
+constexpr int kGemmMinTileRows = SESSD_GEMM_MIN_TILE_ROWS;  // smallest capacity of any kernel: bounds the tile count
 constexpr int kGemmMaxOffsets = 27;  // kernel volumes the rulebook holds (3 x 3 x 3)
 struct TilePlan {
     int count;   // tiles
     int height;  // rows per tile when all tiles have the same length
 };
-__host__ __device__ inline TilePlan tile_plan(int n, int num_cu) {
+__host__ __device__ inline TilePlan tile_plan(int n, int num_cu, int target) {
     TilePlan p;
     if (n <= 0) {
         p.count = num_cu;
         p.height = 1;
         return p;
     }
-    const int r = (n + num_cu * kGemmTargetRows - 1) / (num_cu * kGemmTargetRows);
+    const int r = (n + num_cu * target - 1) / (num_cu * target);
     p.count = num_cu * r;
     p.height = (n + p.count - 1) / p.count;
     return p;
 }
+// tile capacity (rows) of the MFMA kernel that serves this layer shape
+int gemm_tile_rows(int cin, int cout, int dtype);
 int gemm_compute_units();
 
 // equal-work tile cuts for the MFMA kernel, written into `region` (tile_cut_bytes() bytes of the layer's
-// workspace; its first word must be zero before the launch and stays zero when there are no active rows)
+// workspace; its first word must be zero before the launch and stays zero when there are no active rows);
+// target_rows >= kGemmMinTileRows is the tile height aimed at
 size_t tile_cut_bytes(int max_voxels);
-int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, void* region,
-                     hipStream_t stream);
+int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, int target_rows,
+                     void* region, hipStream_t stream);
 
 // picks the kernel for the layer shape; returns SESSD_E_UNSUPPORTED for dtype pairs not covered, and when a
 // dense target is set but the layer does not run on the MFMA kernel (see gemm_runs_on_mfma)

@@ -102,6 +102,8 @@ class ConvPluginBase {
         return weights_packed_dev_ != nullptr && !(flags_ & SESSD_FLAG_FORCE_VALU) &&
                in_channel_ * out_channel_ >= SESSD_TILE_CUT_MIN_WORK;
     }
+    // tile height those cuts aim at: the capacity of this layer's own GEMM kernel
+    int tileRows() const;
     int exportRulebook(const int32_t* nbr, const int32_t* num_out, void* scratch,
                        int32_t* indice_pairs, uint32_t* indice_num, hipStream_t stream) const;
     int freeDevice();

@@ -6,7 +6,7 @@
 // row vary between 1 and 27 with the local density of the scene), and the launch lasts as long as the
 // busiest unit.  Here every row gets the weight  pairs(row) + kRowWeight  and the rows are cut where the
 // running sum crosses multiples of W = ceil(total / T), T = the tile count the equal-length rule would
-// use (tile_plan()).  The constant keeps sparse runs from growing far beyond the kernel's tile capacity;
+// use (tile_plan() with the target height the caller names).  The constant keeps sparse runs from growing far beyond the kernel's tile capacity;
 // runs that still do are walked in capacity-sized pieces by the kernel, so any cut is correct.
 //
 // Two launches over the rows:
@@ -28,7 +28,7 @@ constexpr int kBlock = 256;
 #endif
 constexpr int kRowWeight = SESSD_TILE_ROW_WEIGHT;
 
-__host__ __device__ inline int max_tiles(int max_voxels) { return max_voxels / kGemmTargetRows + 1024 + 1; }
+__host__ __device__ inline int max_tiles(int max_voxels) { return max_voxels / kGemmMinTileRows + 1024 + 1; }
 
 // 256 rows per block, four threads per row (each sums every fourth offset): 1024 threads
 constexpr int kSplit = 4;
@@ -71,7 +71,7 @@ tile_weights(const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_ou
 }
 
 __global__ void __launch_bounds__(kBlock)
-tile_cuts(const int32_t* __restrict__ num_out, int max_voxels, int num_cu, const int32_t* __restrict__ w,
+tile_cuts(const int32_t* __restrict__ num_out, int max_voxels, int num_cu, int target, const int32_t* __restrict__ w,
           const int32_t* __restrict__ bsum, int32_t* __restrict__ hdr) {
     __shared__ int32_t s_before[kBlock / 64], s_total[kBlock / 64], s_wave[kBlock / 64];
     int n = *num_out;
@@ -111,7 +111,7 @@ tile_cuts(const int32_t* __restrict__ num_out, int max_voxels, int num_cu, const
     total = s_total[0] + s_total[1] + s_total[2] + s_total[3];
     for (int v = 0; v < wave; ++v) before += s_wave[v];
     const int excl = before + inc - mine;  // weight of all rows before this one
-    const int tiles = tile_plan(n, num_cu).count;
+    const int tiles = tile_plan(n, num_cu, target).count;
     const int W = (total + tiles - 1) / tiles;  // >= kRowWeight + 1 > 0
     if (row < n) {
         const int id = excl / W;
@@ -134,14 +134,15 @@ size_t tile_cut_bytes(int max_voxels) {
     return align_up(ints * sizeof(int32_t));
 }
 
-int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, void* region,
-                     hipStream_t stream) {
+int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, int target_rows,
+                     void* region, hipStream_t stream) {
+    if (target_rows < kGemmMinTileRows) return fail(SESSD_E_INVALID, "tile cuts: target of %d rows is below %d", target_rows, kGemmMinTileRows);
     int32_t* hdr = static_cast<int32_t*>(region);
     int32_t* w = hdr + 4 + max_tiles(max_voxels) + 1;
     int32_t* bsum = w + max_voxels;
     const int blocks = ceil_div(max_voxels, kBlock);
     hipLaunchKernelGGL(tile_weights, dim3(blocks), dim3(kBlock * kSplit), 0, stream, nbr, num_out, max_voxels, K, w, bsum);
-    hipLaunchKernelGGL(tile_cuts, dim3(blocks), dim3(kBlock), 0, stream, num_out, max_voxels, gemm_compute_units(), w,
+    hipLaunchKernelGGL(tile_cuts, dim3(blocks), dim3(kBlock), 0, stream, num_out, max_voxels, gemm_compute_units(), target_rows, w,
                        bsum, hdr);
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;
