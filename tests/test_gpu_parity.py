@@ -312,6 +312,41 @@ def test_subm_shared_rulebook_skip_pad_and_empty():
     assert np.all(to_np(y0) == 0) and np.all(to_np(num) == 0) and np.all(to_np(pairs) == -1)
 
 
+@pytest.mark.parametrize("owner_cout,sharer_cout", [(64, 32), (32, 64)])
+def test_shared_rulebook_between_layers_of_different_tile_capacity(owner_cout, sharer_cout):
+    """The FP16 32->64 kernel owns up to 64 rows per tile, the 32->32 one 48, and a rulebook's tile cuts aim at
+    the capacity of the layer that built it.  15 000 rows on 256 compute units give runs of ~59 rows under a
+    64-row target: the 48-row kernel has to walk them in two pieces; in the other direction the 64-row kernel
+    runs on cuts made for 48."""
+    grid = (21, 400, 352)
+    n, mv, cin = 15000, 16384, 32
+    rng = np.random.default_rng(41)
+    coors = F.clustered_active_voxels(n, grid, 2, n_blobs=120)
+    feat = O.round_to_half(rng.uniform(-1, 1, (n, cin)).astype(np.float32))
+    w1 = O.round_to_half(rng.normal(0, 0.1, (27, cin, owner_cout)).astype(np.float32))
+    w2 = O.round_to_half(rng.normal(0, 0.1, (27, cin, sharer_cout)).astype(np.float32))
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = np.zeros((mv, cin), np.float32)
+    fbuf[:n] = feat
+    a = api.SubmConv3d(cin, owner_cout, grid[::-1], w1, mv)
+    b = api.SubmConv3d(cin, sharer_cout, grid[::-1], w2, mv)
+    d_feat, d_coors, d_num = dev(fbuf, torch.float16), dev(cbuf), dev(np.array([n], np.int32))
+    y1 = a(d_feat, d_coors, d_num, out_dtype=torch.float16)
+    y2 = b(d_feat, d_coors, d_num, out_dtype=torch.float16, rulebook_from=a)
+    torch.cuda.synchronize()
+    o_pairs, o_num, _ = O.subm_rulebook(coors, n, grid[::-1], mv)
+    o1 = O.round_to_half(O.gather_gemm_scatter(feat, w1, o_pairs, o_num, mv))
+    o2 = O.round_to_half(O.gather_gemm_scatter(feat, w2, o_pairs, o_num, mv))
+    assert_features_close(to_np(y1.float()), o1, RTOL_FP16, "owner %d" % owner_cout)
+    assert_features_close(to_np(y2.float()), o2, RTOL_FP16, "sharer %d" % sharer_cout)
+    # the sharer on its own rulebook (cuts for its own capacity): the same values up to the order in which the
+    # offsets of a row are summed, which follows the tile the row falls in
+    y3 = b(d_feat, d_coors, d_num, out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    assert_features_close(to_np(y2.float()), to_np(y3.float()), 2e-3, "shared vs own cuts")
+
+
 def test_subm_bad_coordinate_is_flagged_not_written():
     grid = (5, 20, 20)
     coors = np.array([[0, 1, 1, 1], [0, 1, 1, 2], [0, 7, 1, 1], [0, 1, 25, 1]], np.int32)   # rows 2,3 outside
