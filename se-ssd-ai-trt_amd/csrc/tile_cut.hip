@@ -112,12 +112,16 @@ tile_cuts(const int32_t* __restrict__ num_out, int max_voxels, int num_cu, int t
     for (int v = 0; v < wave; ++v) before += s_wave[v];
     const int excl = before + inc - mine;  // weight of all rows before this one
     const int tiles = tile_plan(n, num_cu, target).count;
-    const int W = (total + tiles - 1) / tiles;  // >= kRowWeight + 1 > 0
+    // W is kept above the heaviest possible row: a row then advances the tile id by at most one, so every id
+    // up to the last gets its start written (with few rows -- fewer than tiles -- total / tiles would fall
+    // below a row's weight, ids would skip, and the skipped entries of the table would be read unwritten)
+    int W = (total + tiles - 1) / tiles;
+    W = W > kGemmMaxOffsets + kRowWeight ? W : kGemmMaxOffsets + kRowWeight + 1;
     if (row < n) {
         const int id = excl / W;
         const int prev = row == 0 ? -1 : (excl - w[row - 1]) / W;
         int32_t* start = hdr + 4;
-        if (id != prev) start[id] = row;  // a row weighs less than W: ids grow by at most one per row
+        if (id != prev) start[id] = row;  // ids grow by at most one per row (W exceeds every row weight)
         if (row == n - 1) {
             start[id + 1] = n;
             hdr[1] = W;

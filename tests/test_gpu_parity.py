@@ -347,6 +347,54 @@ def test_shared_rulebook_between_layers_of_different_tile_capacity(owner_cout, s
     assert_features_close(to_np(y2.float()), to_np(y3.float()), 2e-3, "shared vs own cuts")
 
 
+@pytest.mark.parametrize("n", [1, 17, 300])
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+def test_fewer_rows_than_tiles_in_a_wide_layer(n, dtype):
+    """A handful of active rows in a layer wide enough to get equal-work tile cuts: the rows weigh more than
+    total / tiles, and every entry of the cut table up to the last tile must still be written."""
+    grid = (3, 48, 15)
+    mv, cin, cout = n + 225, 64, 64
+    half = dtype == "fp16"
+    rng = np.random.default_rng(n)
+    coors = F.clustered_active_voxels(n, grid, 5, n_blobs=2)
+    feat = rng.uniform(-1, 1, (n, cin)).astype(np.float32)
+    w = rng.normal(0, 0.1, (27, cin, cout)).astype(np.float32)
+    if half:
+        feat, w = O.round_to_half(feat), O.round_to_half(w)
+    conv = api.SubmConv3d(cin, cout, grid[::-1], w, mv)
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = np.zeros((mv, cin), np.float32)
+    fbuf[:n] = feat
+    tdt = torch.float16 if half else torch.float32
+    for _ in range(2):                                       # the second call finds the first one's table
+        out = conv(dev(fbuf, tdt), dev(cbuf), dev(np.array([n], np.int32)), out_dtype=tdt)
+        torch.cuda.synchronize()
+        o_pairs, o_num, _ = O.subm_rulebook(coors, n, grid[::-1], mv)
+        o_out = O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv)
+        if half:
+            assert_features_close(to_np(out.float()), O.round_to_half(o_out), RTOL_FP16, "few rows fp16")
+        else:
+            assert_features_close(to_np(out), o_out, RTOL_FP32, "few rows fp32")
+        assert conv.status() == 0
+
+
+def test_few_output_sites_in_a_wide_strided_layer():
+    """36 input cells, kernel (3,3,1), stride (3,1,2): a few dozen output rows in a 32 -> 64 layer."""
+    k, s, p, ig = (3, 3, 1), (3, 1, 2), (0, 1, 0), (3, 26, 7)
+    og = tuple(B.conv_out_size(ig[a], k[a], s[a], p[a]) for a in range(3))
+    layer = B.Layer("t", D.SESSD_LAYER_SPARSE, 32, 64, og[::-1], k, s, p)
+    n, mv = 36, 86
+    rng = np.random.default_rng(4)
+    coors = F.random_active_voxels(n, ig, 11)
+    feat = rng.uniform(-1, 1, (n, 32)).astype(np.float32)
+    w = rng.normal(0, 0.1, (layer.kvol, 32, 64)).astype(np.float32)
+    conv, out, oc, on, pairs, num = run_sparse(layer, coors, n, feat, w, mv, ig)
+    o_pairs, o_num, o_oc, o_on, o_st = O.sparse_rulebook(coors, n, og[::-1], k, s, p, mv)
+    assert on == o_on and conv.status() == o_st and np.array_equal(oc, o_oc) and np.array_equal(num, o_num)
+    assert_features_close(out, O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), RTOL_FP32, "few output sites")
+
+
 def test_subm_bad_coordinate_is_flagged_not_written():
     grid = (5, 20, 20)
     coors = np.array([[0, 1, 1, 1], [0, 1, 1, 2], [0, 7, 1, 1], [0, 1, 25, 1]], np.int32)   # rows 2,3 outside
