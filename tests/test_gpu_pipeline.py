@@ -145,6 +145,36 @@ def test_overlapped_graph_schedule_with_reference_pad_rows():
         assert np.array_equal(rows[0][0][cnt:], np.broadcast_to(want_pad, (mv - cnt, len(want_pad)))), layers[l].name
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+def test_tiny_frames_through_the_pipeline(dtype):
+    """Frames of 0, 1, 7, 40 and 150 points through one pipeline (overlapped schedule, captured graph): the wide
+    layers then see far fewer rows than they have tiles.  Site counts exact, dense tensor against the oracle."""
+    layers = B.reference_layers()
+    W = B.random_weights(layers, seed=3, w_std=0.05)
+    half = dtype == "fp16"
+    if half:
+        W = half_weights(W)
+    mp, mv = 1024, 4096
+    pipe = api.Pipeline(layers, W, mp, mv, feature_dtype=dtype, share_rulebooks=True, skip_pad_rows=True,
+                        use_graph=True, overlap_streams=True)
+    p, n = points_input(np.zeros((0, 4), np.float32), mp)
+    dense, stream = pipe.new_dense(), torch.cuda.Stream()
+    for npts in (150, 0, 1, 40, 7):
+        pts = F.lidar_frame(npts, 100 + npts) if npts else np.zeros((0, 4), np.float32)
+        hp, hn = points_input(pts, mp)
+        with torch.cuda.stream(stream):
+            p.copy_(hp)
+            n.copy_(hn)
+            pipe.enqueue(p, n, dense, stream)
+        stream.synchronize()
+        ref = O.frame(pts, B.voxelgen_desc(max_voxels=mv), layers, W, B.dense_desc(), round_half=half)
+        assert pipe.status() == ref["status"] == 0
+        for l in range(-1, len(layers)):
+            assert pipe.layer_count(l) == ref["counts"][l + 1], (npts, l)
+        assert_features_close(to_np(dense).astype(np.float32), ref["dense"], 10 * RTOL_FP16 if half else RTOL_END_TO_END,
+                              "dense, %d points" % npts)
+
+
 def test_full_backbone_config3_frame_and_graph_replay():
     """Benchmark configuration 3: the 20 000-point frame (~17 k voxels) through the reference's 14 conv layers.
     The eager enqueue and repeated replays of the captured graph must give identical bits."""
