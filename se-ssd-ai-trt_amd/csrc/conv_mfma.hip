@@ -198,11 +198,14 @@ conv_mfma(const T* __restrict__ in, TO* __restrict__ out, const void* __restrict
     const int kgrp = wave / CS;   // offsets are dealt to this group ...
     const int chalf = wave % CS;  // ... and this wave computes this part of their columns
     constexpr int kVecPerRow = COUT / 4;
-    // scale/shift are fetched now, into LDS, so that the epilogue does not wait for global memory
+    // scale/shift are requested now and parked in LDS (below, once the first piece's list loads are out as
+    // well, so that the workgroup waits once for all of them): the epilogue does not wait for global memory
     __shared__ float s_epi[2 * COUT];
-    for (int c = tid; c < COUT; c += kWaves * 64) {
-        s_epi[c] = scale ? scale[c] : 1.f;
-        s_epi[COUT + c] = shift ? shift[c] : 0.f;
+    static_assert(COUT <= kWaves * 64, "one thread per output channel fetches the epilogue constants");
+    float epi_scale = 1.f, epi_shift = 0.f;
+    if (tid < COUT) {
+        if (scale) epi_scale = scale[tid];
+        if (shift) epi_shift = shift[tid];
     }
     const int ec4 = (tid % kVecPerRow) * 4;  // this thread's epilogue columns, the same for every row it stores
     static_assert((kWaves * 64) % kVecPerRow == 0, "a thread must keep its columns from row to row");
@@ -252,6 +255,10 @@ conv_mfma(const T* __restrict__ in, TO* __restrict__ out, const void* __restrict
     for (int s = 0; s < kListsPerWave; ++s) {
         const int k = wave + s * kWaves;
         staged[s] = (k < K && lane < rows) ? nbr[(size_t)k * max_voxels + row0 + lane] : -1;
+    }
+    if (row0 == run_begin && tid < COUT) {
+        s_epi[tid] = epi_scale;
+        s_epi[COUT + tid] = epi_shift;
     }
 #pragma unroll
     for (int s = 0; s < kListsPerWave; ++s) {
