@@ -40,7 +40,7 @@ def profiled_traffic(kernel, dtype):
             for line in f:
                 cells = [c.strip() for c in line.split("|")]
                 if len(cells) >= 8 and cells[1] == kernel and cells[2].isdigit():
-                    return (float(cells[5]) + float(cells[6])) * 1e6
+                    return float(round((float(cells[5]) + float(cells[6])) * 1e6))
     except (OSError, ValueError):
         pass
     return None
