@@ -28,6 +28,38 @@ def test_struct_layouts_match_header_sizes():
     assert C.sizeof(D.LayerSpec) == 12 + 12 * 4
 
 
+def test_header_compiles_as_c_and_the_ctypes_mirror_matches_it(tmp_path):
+    """include/sessd3d.h is a C header (C99, -pedantic): a C program built against it prints the size of every
+    struct and the offset of every field, and the ctypes mirror the tests and the benchmark bind with must
+    agree field by field."""
+    import os
+    import shutil
+    import subprocess
+    if not shutil.which("gcc"):
+        pytest.skip("no C compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    pairs = [("sessd_tensor_desc", D.TensorDesc), ("sessd_voxelgen_desc", D.VoxelGenDesc),
+             ("sessd_submconv3d_desc", D.SubmConv3dDesc), ("sessd_sparseconv3d_desc", D.SparseConv3dDesc),
+             ("sessd_sparse2dense_desc", D.Sparse2DenseDesc), ("sessd_layer_spec", D.LayerSpec),
+             ("sessd_pipeline_desc", D.PipelineDesc)]
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "sessd3d.h"', 'int main(void) {']
+    for cname, mirror in pairs:
+        lines.append('    printf("%s %%zu\\n", sizeof(%s));' % (cname, cname))
+        for fname, _ in mirror._fields_:
+            lines.append('    printf("%s.%s %%zu\\n", offsetof(%s, %s));' % (cname, fname, cname, fname))
+    lines += ['    return 0;', '}']
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines) + "\n")
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(root, "include"),
+                    str(src), "-o", str(exe)], check=True)
+    out = dict(l.split() for l in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    for cname, mirror in pairs:
+        assert int(out[cname]) == C.sizeof(mirror), cname
+        for fname, _ in mirror._fields_:
+            assert int(out["%s.%s" % (cname, fname)]) == getattr(mirror, fname).offset, (cname, fname)
+
+
 def test_reference_backbone_table_matches_python_table():
     L = api.lib()
     specs = (D.LayerSpec * 14)()
