@@ -28,11 +28,12 @@ def sources():
 
 
 def headers():
-    return sorted(glob.glob(os.path.join(SRC_DIR, "*.h"))) + [os.path.join(HERE, "..", "include", "sessd3d.h")]
+    return (sorted(glob.glob(os.path.join(SRC_DIR, "*.h"))) + [os.path.join(HERE, "..", "include", "sessd3d.h")] +
+            [os.path.join(HERE, "examples", "run_frame.c")])
 
 
 def is_stale():
-    if not os.path.exists(LIB):
+    if not os.path.exists(LIB) or not os.path.exists(os.path.join(HERE, "lib", "run_frame")):
         return True
     t = os.path.getmtime(LIB)
     return any(os.path.getmtime(p) > t for p in sources() + headers())
@@ -64,7 +65,26 @@ def build(force=True, jobs=8, verbose=False):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stdout)
+    build_example()
     return LIB
+
+
+EXAMPLE_SRC = os.path.join(HERE, "examples", "run_frame.c")
+EXAMPLE = os.path.join(HERE, "lib", "run_frame")
+
+
+def build_example():
+    """The C host of the library (examples/run_frame.c): plain C99 with gcc against include/sessd3d.h and the
+    HIP runtime API, linked to the library beside it."""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [os.environ.get("CC", "gcc"), "-std=c99", "-O2", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__",
+           "-I", os.path.join(HERE, "..", "include"), "-I", os.path.join(rocm, "include"), EXAMPLE_SRC, "-o", EXAMPLE,
+           "-L", os.path.dirname(LIB), "-lsessd3d", "-L", os.path.join(rocm, "lib"), "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building the C example failed:\n" + r.stdout)
+    return EXAMPLE
 
 
 if __name__ == "__main__":

@@ -68,3 +68,31 @@ def test_frame_harness_over_a_directory(tmp_path, capsys):
         _, _, n, _, _ = O.voxelize(pts, B.POINT_CLOUD_RANGE, B.VOXEL_SIZE, 5, 16384)
         assert rec["points"] == len(pts) and rec["voxels"] == n and rec["status"] == 0
         assert rec["ms_with_h2d"] >= rec["ms_pipeline"] > 0
+
+
+def test_c_host_program_matches_the_python_binding(tmp_path):
+    """examples/run_frame.c -- a C99 program on the C-ABI and the HIP runtime API alone: frame file in, weight
+    file in, dense tensor out -- against the ctypes binding on the same two files: same voxel count, same status,
+    the same dense tensor bit for bit."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(__file__), "..", "se-ssd-ai-trt_amd", "lib", "run_frame")
+    if not os.path.exists(exe):
+        pytest.skip("se-ssd-ai-trt_amd/lib/run_frame is not built (python se-ssd-ai-trt_amd/build.py)")
+    layers = B.reference_layers()
+    wts = tmp_path / "sessd.wts"
+    B.write_wts(wts, B.random_state_dict(layers, seed=15, w_std=0.05))
+    pts = F.lidar_frame(9000, 6)
+    frame = tmp_path / "000000.bin"
+    np.ascontiguousarray(pts, np.float32).tofile(frame)
+    out = tmp_path / "dense.bin"
+    r = subprocess.run([exe, str(frame), str(wts), str(out), "3"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    words = r.stdout.split()
+    rec = dict(zip(words[::2], words[1::2]))
+    pipe = api.Pipeline(layers, api.WeightFile(path=str(wts)), 80000, B.MAX_VOXELS, share_rulebooks=True,
+                        skip_pad_rows=True, use_graph=True, overlap_streams=True)
+    dense = run(pipe, pts, 80000)
+    assert int(rec["points"]) == len(pts) and int(rec["voxels"]) == pipe.layer_count(-1)
+    assert int(rec["status"]) == pipe.status() == 0 and float(rec["ms_per_frame"]) > 0
+    got = np.fromfile(out, np.float32).reshape(tuple(dense.shape))
+    assert got.any() and np.array_equal(got, to_np(dense))
