@@ -8,9 +8,8 @@ for p in (os.path.join(ROOT, "se-ssd-ai-trt_amd"), os.path.join(ROOT, "tests")):
     if p not in sys.path:
         sys.path.insert(0, p)
 
-# Real frames the reference ships; only present in the authoring container.  Tests that read them
-# are CPU tests and skip when the directory is absent.
-KITTI_DIR = "/root/reference/data/kitti_training_velodyne_reduced"
+# The first frame of the reference's data directory, kept as a fixture (tests/golden/README.md).
+KITTI_FRAME0 = os.path.join(ROOT, "tests", "golden", "kitti_000000.bin")
 
 
 def pytest_configure(config):
@@ -20,7 +19,4 @@ def pytest_configure(config):
 @pytest.fixture(scope="session")
 def kitti_frame0():
     import numpy as np
-    path = os.path.join(KITTI_DIR, "000000.bin")
-    if not os.path.exists(path):
-        pytest.skip("KITTI fixture frames not present")
-    return np.fromfile(path, np.float32).reshape(-1, 4)
+    return np.fromfile(KITTI_FRAME0, np.float32).reshape(-1, 4)

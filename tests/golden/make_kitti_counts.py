@@ -1,6 +1,6 @@
 """Recompute tests/golden/kitti_000000_counts.json with numpy only (no oracle, no reference code).
 
-Reads frame 000000 from the reference's data directory, voxelises it in float32, and walks the four
+Reads frame 000000 of the reference's data directory (kept beside this script as kitti_000000.bin), voxelises it in float32, and walks the four
 strided stages with set arithmetic: an output cell o of a sparse layer is active iff some active
 input cell c satisfies c = o*s - p + k for an offset 0 <= k < ksize on every axis; the pairs of a
 layer are all (input, output, offset) triples that satisfy it.
@@ -11,7 +11,7 @@ import sys
 
 import numpy as np
 
-SRC = "/root/reference/data/kitti_training_velodyne_reduced/000000.bin"
+SRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "kitti_000000.bin")
 
 
 def voxelize(p):

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import oracle_lib as O
-from gpu_util import RTOL_FP16, RTOL_FP32, assert_features_close, canonical, points_input, to_np
+from gpu_util import RTOL_END_TO_END, RTOL_FP16, RTOL_FP32, assert_features_close, canonical, points_input, to_np
 from sessd3d import api, backbone as B, ctypes_defs as D, frames as F
 
 pytestmark = pytest.mark.gpu
@@ -20,12 +20,6 @@ def run_pipeline(pts, layers, W, max_points, max_voxels, **kw):
         pipe.enqueue(p, n, dense, stream)
     stream.synchronize()
     return pipe, dense, (p, n, stream)
-
-
-# End to end the FP32 rounding differences of 14 stacked layers compound (each layer's error is amplified
-# by the next layer's weights and by cancellation), so the whole-frame comparison uses 1e-3; the 1e-4
-# bound is checked layer by layer, each layer of the oracle being fed the GPU's own input rows.
-RTOL_END_TO_END = 1e-3
 
 
 def compare_with_oracle(pipe, dense, pts, layers, W, max_voxels, rtol_layer, rtol_frame=RTOL_END_TO_END):

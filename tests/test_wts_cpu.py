@@ -120,11 +120,8 @@ def test_load_frame_reads_kitti_layout(tmp_path):
     assert api.load_frame(str(empty), 10)[1] == 0
 
 
-def test_load_frame_on_the_reference_fixture_when_present():
-    import os
-    path = "/root/reference/data/kitti_training_velodyne_reduced/000000.bin"
-    if not os.path.exists(path):
-        pytest.skip("the reference checkout is not on this machine")
-    want = np.fromfile(path, np.float32).reshape(-1, 4)
-    buf, n = api.load_frame(path, B.MAX_POINTS)
-    assert n == len(want) and np.array_equal(buf[:n], want)
+def test_load_frame_on_the_reference_fixture(kitti_frame0):
+    """The first frame of the reference's data directory (kept under tests/golden): 20 285 points."""
+    from conftest import KITTI_FRAME0
+    buf, n = api.load_frame(KITTI_FRAME0, B.MAX_POINTS)
+    assert n == len(kitti_frame0) == 20285 and np.array_equal(buf[:n], kitti_frame0)
