@@ -121,6 +121,20 @@ size_t sessd_voxelgen_workspace_size(const sessd_voxelgen* h, const sessd_tensor
 int sessd_voxelgen_enqueue(sessd_voxelgen* h, const sessd_tensor_desc* inDesc,
                            const sessd_tensor_desc* outDesc, const void* const* inputs,
                            void* const* outputs, void* workspace, sessd_stream_t stream);
+/* No counterpart in the reference.  For callers that cannot allocate device memory or hand over a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * sessd_voxelgen_enqueue without the workspace argument.  The scratch memory is a static device array
+ * inside the library, 8 MiB on every GPU the library runs on, held until the process ends; that is
+ * enough for the reference's shape (80000-row points tensor, 5 points per voxel: 7.7 MB) and a request
+ * that needs more is rejected with SESSD_E_INVALID before anything is launched.  The call allocates and
+ * frees nothing; its first use on a device looks the array's address up (make that call outside a
+ * stream capture).  All calls on one GPU share the array: it is cleared by each call, and two calls that
+ * overlap in time on one GPU (different streams, different handles) race.  Outputs are bit-identical
+ * to sessd_voxelgen_enqueue's. */
+int sessd_voxelgen_enqueue_static(sessd_voxelgen* h, const sessd_tensor_desc* inDesc,
+                                  const sessd_tensor_desc* outDesc, const void* const* inputs,
+                                  void* const* outputs, sessd_stream_t stream);
+/* workspace NULL = the static scratch of sessd_voxelgen_enqueue_static on the current device */
 int sessd_voxelgen_status(const sessd_voxelgen* h, const void* workspace, sessd_stream_t stream,
                           int32_t* status);
 int sessd_voxelgen_set_flags(sessd_voxelgen* h, int32_t flags);

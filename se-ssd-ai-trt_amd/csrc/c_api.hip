@@ -75,9 +75,19 @@ int sessd_voxelgen_enqueue(sessd_voxelgen* h, const sessd_tensor_desc* inDesc, c
     NEED(h, "null handle");
     return H_VG(h)->enqueue(inDesc, outDesc, inputs, outputs, workspace, static_cast<hipStream_t>(stream));
 }
+int sessd_voxelgen_enqueue_static(sessd_voxelgen* h, const sessd_tensor_desc* inDesc, const sessd_tensor_desc* outDesc,
+                                  const void* const* inputs, void* const* outputs, sessd_stream_t stream) {
+    NEED(h, "null handle");
+    return H_VG(h)->enqueueStatic(inDesc, outDesc, inputs, outputs, static_cast<hipStream_t>(stream));
+}
 int sessd_voxelgen_status(const sessd_voxelgen* h, const void* workspace, sessd_stream_t stream, int32_t* status) {
-    NEED(h && workspace && status, "null argument");
+    NEED(h && status, "null argument");
     NEED(CH_VG(h)->lastMaxPoints_ > 0, "configure or enqueue must run first (the layout depends on max_points)");
+    void* own = nullptr;
+    if (!workspace) {  // the static scratch of sessd_voxelgen_enqueue_static on the current device
+        SESSD_TRY(voxelgen_static_scratch(&own));
+        workspace = own;
+    }
     return read_status_word(workspace, CH_VG(h)->statusOffset(CH_VG(h)->lastMaxPoints_),
                             static_cast<hipStream_t>(stream), status);
 }

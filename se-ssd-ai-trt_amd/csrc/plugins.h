@@ -31,6 +31,10 @@ class VoxelGeneratorPlugin {
     int enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
                 const void* const* inputs, void* const* outputs, void* workspace,
                 hipStream_t stream);
+    // enqueue() on the library's own static scratch array instead of a caller's workspace: allocates nothing;
+    // rejects points tensors whose layout does not fit the array.  Calls that overlap on one GPU race.
+    int enqueueStatic(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
+                      const void* const* inputs, void* const* outputs, hipStream_t stream);
     size_t getSerializationSize() const;
     void serialize(void* buffer) const;
     size_t statusOffset(int max_points) const;
@@ -244,6 +248,8 @@ inline T readFromBuffer(const char*& buffer) {
 }
 
 int read_status_word(const void* workspace, size_t offset, hipStream_t stream, int32_t* status);
+// device address of the voxelizer's static scratch array on the current device (voxel_generator.hip)
+int voxelgen_static_scratch(void** out);
 
 // helpers shared by the two conv plugins (conv_base.hip)
 int conv_check_io(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,

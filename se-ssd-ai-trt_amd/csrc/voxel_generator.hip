@@ -16,6 +16,8 @@
 // The result equals a sequential walk over the points: ids in first-appearance order, the first S
 // points of a cell kept, cells first seen after max_voxels dropped.  All traffic is O(points):
 // 16 B/point read + 32 B/voxel written, plus the hash clear.
+#include <mutex>
+
 #include "plugins.h"
 
 namespace sessd {
@@ -376,6 +378,53 @@ int read_status_word(const void* workspace, size_t offset, hipStream_t stream, i
                                  hipMemcpyDeviceToHost, stream));
     SESSD_HIP_TRY(hipStreamSynchronize(stream));
     return SESSD_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The enqueue that allocates nothing and takes no workspace: its scratch memory is a file-scope device
+// array.  Every GPU the library runs on holds its own copy of the array (8 MiB, until the process ends)
+// at its own address; `scratch` below is only the host-side name of the symbol, never a device pointer,
+// so host code asks the runtime for the address once per device and hands THAT to the kernels.
+// ---------------------------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = 8u << 20;  // fits the reference's 80000-point tensor (7.7 MB)
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};  // device address of `scratch`, per device
+}  // namespace
+
+// -> address of the current device's copy of `scratch` (resolved on the first call per device)
+int voxelgen_static_scratch(void** out) {
+    int dev = -1;
+    SESSD_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(SESSD_E_UNSUPPORTED, "voxelgen: device index %d is beyond %d", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        SESSD_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(SESSD_E_HIP, "voxelgen: the static scratch array has no address on device %d", dev);
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return SESSD_OK;
+}
+
+int VoxelGeneratorPlugin::enqueueStatic(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
+                                        const void* const* inputs, void* const* outputs, hipStream_t stream) {
+    if (!inputDesc || inputDesc[0].nbDims != 3 || inputDesc[0].d[1] <= 0)
+        return fail(SESSD_E_INVALID, "voxelgen.enqueue_static: points must be [1,max_points,F]");
+    // the size check comes before any runtime call: a request that does not fit touches nothing
+    const size_t need = carve(nullptr, inputDesc[0].d[1]).total;
+    if (need > kStaticScratchBytes)
+        return fail(SESSD_E_INVALID,
+                    "voxelgen.enqueue_static: a points tensor of %d rows with %d points per voxel needs %zu bytes of "
+                    "scratch, the static buffer holds %zu; use sessd_voxelgen_enqueue with a workspace of your own",
+                    inputDesc[0].d[1], pointNum_, need, kStaticScratchBytes);
+    void* ws = nullptr;
+    SESSD_TRY(voxelgen_static_scratch(&ws));
+    return enqueue(inputDesc, outputDesc, inputs, outputs, ws, stream);
 }
 
 }  // namespace sessd

@@ -69,6 +69,7 @@ def lib():
         getattr(L, "sessd_%s_export_rulebook" % name).argtypes = [vp, vp, vp, vp, vp]
     L.sessd_voxelgen_create.argtypes = [C.POINTER(D.VoxelGenDesc), VPP]
     L.sessd_voxelgen_grid_size.argtypes = [vp, C.POINTER(i32)]
+    L.sessd_voxelgen_enqueue_static.argtypes = [vp, TD, TD, VPP, VPP, vp]
     L.sessd_submconv3d_create.argtypes = [C.POINTER(D.SubmConv3dDesc), vp, VPP]
     L.sessd_submconv3d_enqueue_shared.argtypes = [vp, TD, TD, VPP, VPP, vp, vp]
     L.sessd_sparseconv3d_create.argtypes = [C.POINTER(D.SparseConv3dDesc), vp, VPP]
@@ -226,6 +227,16 @@ class VoxelGenerator(_Plugin):
         g = (C.c_int32 * 3)()
         check(lib().sessd_voxelgen_grid_size(self.h, g))
         return tuple(g)
+
+    def enqueue_static(self, inputs, outputs, stream=None):
+        """enqueue() on the library's static scratch array: no workspace, no allocation (sessd_voxelgen_enqueue_static)."""
+        check(lib().sessd_voxelgen_enqueue_static(self.h, _descs(inputs), _descs(outputs), _voidpp(inputs),
+                                                  _voidpp(outputs), _stream_ptr(stream)))
+
+    def status_static(self, stream=None) -> int:
+        s = C.c_int32(0)
+        check(lib().sessd_voxelgen_status(self.h, None, _stream_ptr(stream), C.byref(s)))
+        return s.value
 
     def __call__(self, points, points_size, stream=None):
         """points f32[max_points,F], points_size i32[1] (device) -> voxels, coors, voxel_num (device)"""
