@@ -105,6 +105,24 @@ def test_voxelgen_host_side():
     assert b"null" in L.sessd_last_error()
 
 
+def test_voxelgen_static_enqueue_rejects_oversize_before_any_gpu_call():
+    """sessd_voxelgen_enqueue_static: a points tensor whose scratch layout exceeds the library's static 8 MiB array
+    is refused with a message that names both sizes, before any runtime call (so it is testable without a GPU)."""
+    vg = api.VoxelGenerator(max_voxels=60000)
+    L = api.lib()
+    ind = (D.TensorDesc * 2)(D.TensorDesc.make([1, 150000, 4], D.SESSD_FLOAT), D.TensorDesc.make([1], D.SESSD_INT32))
+    outd = (D.TensorDesc * 3)(D.TensorDesc.make([1, 60000, 4], D.SESSD_FLOAT),
+                              D.TensorDesc.make([1, 60000, 4], D.SESSD_INT32), D.TensorDesc.make([1], D.SESSD_INT32))
+    fake = (C.c_void_p * 3)(16, 32, 48)                       # never dereferenced: the call fails first
+    assert L.sessd_voxelgen_workspace_size(vg.h, ind, 2, outd, 3) > 8 * 2 ** 20
+    assert L.sessd_voxelgen_enqueue_static(vg.h, ind, outd, fake, fake, None) == D.SESSD_E_INVALID
+    msg = L.sessd_last_error()
+    assert b"static buffer holds 8388608" in msg and b"150000" in msg
+    ind[0] = D.TensorDesc.make([1, 80000, 4], D.SESSD_FLOAT)  # the reference's shape fits
+    assert L.sessd_voxelgen_workspace_size(vg.h, ind, 2, outd, 3) <= 8 * 2 ** 20
+    assert L.sessd_voxelgen_enqueue_static(None, ind, outd, fake, fake, None) == D.SESSD_E_INVALID
+
+
 def test_voxelgen_create_rejects_bad_fields():
     L = api.lib()
     d = B.voxelgen_desc()
