@@ -1,15 +1,25 @@
 #!/usr/bin/env python3
 """Benchmark of the 3-D front end on one MI355X: voxelGenerator -> SpMiddleFHD conv stack -> sparse2Dense.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--points 20000] [--seed 0] [--dtype fp32|fp16]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3|4|5] [--seed 0]
 
 A "step" is one frame: one pass of the whole path over one seeded synthetic LiDAR frame that is already
 resident in device memory.  The timed region is exactly K pipeline enqueues bracketed by device
-synchronisation.  One JSON line is printed with the frame time, the roofline position of the dominant
-kernel (the 64->64 channel gather-GEMM, timed with HIP events on the pipeline's stream) and the CPU
-baseline (the scalar oracle port, one core, same frame).
+synchronisation.  One JSON line is printed:
+
+  value / ms_per_step  ms per frame of the headline configuration (3: 20 000 points, FP32), back-to-back graph launches
+  roofline             the dominant kernel (the 64->64 channel gather-GEMM), timed live with HIP events on the
+                       pipeline's stream, against the FP32 matrix peak
+  parity               the timed configuration's tensors against the CPU oracle on the same frame (sites and their
+                       numbering bit-exact, features per layer within 1e-4, end to end bounded by an FP64
+                       recomputation); a mismatch makes the run exit non-zero
+  other_configs        configurations 4 (60 000 points, voxel cap 40 000, FP16) and 5 (150 000 points over 360
+                       degrees, voxel cap 60 000, doubled widths, FP16; p10/p50/p90 over seeded frames) and the
+                       reference's first KITTI frame: ms/frame, dominant-kernel roofline, parity
+  cpu_baseline         the CPU port (the parity oracle) on the same frame, on the host's cores
 """
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -22,6 +32,11 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 PEAK_FP32_TFLOPS = 157.3    # MI355X dense FP32 (vector and matrix)
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense FP16 MFMA
 
+PRESETS = {3: dict(points=20000, dtype="fp32", max_voxels=60000, voxel_cap=60000, width=1, full=False),
+           4: dict(points=60000, dtype="fp16", max_voxels=100000, voxel_cap=40000, width=1, full=False),
+           5: dict(points=150000, dtype="fp16", max_voxels=200000, voxel_cap=60000, width=2, full=True)}
+KITTI_FRAME0 = os.path.join(ROOT, "tests", "golden", "kitti_000000.bin")
+
 
 def layer_work(layer, n_in, n_out, pairs, esize):
     """Algorithmic work of one conv layer's gather-GEMM launch: flops = 2*P*Cin*Cout; bytes = gathered
@@ -31,19 +46,30 @@ def layer_work(layer, n_in, n_out, pairs, esize):
     return flops, bytes_
 
 
-def profiled_traffic(kernel, dtype):
+def kernel_source_hash():
+    """Short hash of the gather-GEMM kernel's source: the committed counter summaries carry the hash of the source
+    they were collected on, so a figure taken from them can be told from a stale one."""
+    with open(os.path.join(ROOT, "se-ssd-ai-trt_amd", "csrc", "conv_mfma.hip"), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:12]
+
+
+def profiled_traffic(kernel, config, dtype):
     """HBM bytes per launch of `kernel` from the committed rocprofv3 summary (FETCH_SIZE and WRITE_SIZE
-    runs, scaled by a copy kernel of known size), or None when no summary covers it."""
-    path = os.path.join(ROOT, "profiles", "frame_pipeline_config3_%s.md" % dtype)
+    runs, scaled by a copy kernel of known size) -> (bytes or None, whether the summary was collected on the
+    current kernel source)."""
+    path = os.path.join(ROOT, "profiles", "frame_pipeline_config%d_%s.md" % (config, dtype))
+    value, fresh = None, False
     try:
         with open(path) as f:
             for line in f:
+                if line.startswith("kernel source hash"):
+                    fresh = kernel_source_hash() in line
                 cells = [c.strip() for c in line.split("|")]
-                if len(cells) >= 8 and cells[1] == kernel and cells[2].isdigit():
-                    return float(round((float(cells[5]) + float(cells[6])) * 1e6))
+                if len(cells) >= 8 and cells[1] == kernel and cells[2].isdigit() and value is None:
+                    value = float(round((float(cells[5]) + float(cells[6])) * 1e6))
     except (OSError, ValueError):
         pass
-    return None
+    return value, fresh
 
 
 def cpu_model():
@@ -58,14 +84,18 @@ def cpu_model():
     return "unknown CPU"
 
 
-def cpu_baseline(pts, layers, W, max_voxels, voxel_cap, budget_s=24.0):
+def host_threads():
+    # a one-GPU machine of this pool gives a job 16 cores, whatever os.cpu_count() reports
+    return max(1, min(16, os.cpu_count() or 1))
+
+
+def cpu_baseline(pts, layers, W, voxel_cap, budget_s=20.0):
     """The CPU port (the parity oracle) on the same frame, a bounded number of frames: once on one thread and
     once with the pairs of every kernel offset split over the host's cores (same bits either way)."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_lib as O
     from sessd3d import backbone as B
-    # (the oracle uses one capacity for every tensor; the voxelizer's cap equals it in the headline config)
-    vg = B.voxelgen_desc(max_voxels=max_voxels if voxel_cap >= max_voxels else voxel_cap)
+    vg = B.voxelgen_desc(max_voxels=voxel_cap)   # (oracle_frame has one capacity; it equals the layers' in config 3)
     dd = B.dense_desc(channel=layers[-1].cout)
 
     def median_ms(max_frames, budget):
@@ -77,10 +107,10 @@ def cpu_baseline(pts, layers, W, max_voxels, voxel_cap, budget_s=24.0):
         times.sort()
         return times[len(times) // 2], len(times)
 
+    O.set_threads(1)
     O.frame(pts, vg, layers, W, dd)          # warm-up (allocates the dense index grids)
     one, n_one = median_ms(3, budget_s / 2)
-    # a one-GPU machine of this pool gives a job 16 cores, whatever os.cpu_count() reports
-    threads = max(1, min(16, os.cpu_count() or 1))
+    threads = host_threads()
     O.set_threads(threads)
     try:
         O.frame(pts, vg, layers, W, dd)
@@ -95,14 +125,207 @@ def cpu_baseline(pts, layers, W, max_voxels, voxel_cap, budget_s=24.0):
                                                                cpu_model())}
 
 
+def parity_gate(pipe, dense, pts, layers, W, voxel_cap, layer_cap, half):
+    """The tensors of the frame the pipeline last ran against the CPU oracle (tests/gpu_util.py: every layer with the
+    oracle fed the GPU's rows, the oracle's own chain, and an FP64 recomputation).  -> dict with ok = True/False."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib as O
+    import gpu_util as G
+    from sessd3d import backbone as B
+    O.set_threads(host_threads())
+    rep = {}
+    try:
+        G.check_frame_against_oracle(pipe, dense, pts, layers, W, voxel_cap, layer_cap, half, B.DENSE_SIZE_XYZ, rep)
+        ok, why = True, None
+    except AssertionError as e:
+        ok, why = False, str(e)[:400] or "assertion failed"
+    finally:
+        O.set_threads(1)
+    out = {"ok": ok, "checked": "voxel means, coordinates, counts, per-layer output sites + numbering and status words bit-exact; "
+                                "features per layer <= %g relative (oracle fed the GPU's rows); GPU's RMS distance from an FP64 "
+                                "recomputation <= 2x the oracle's, per layer" % (G.RTOL_FP16 if half else G.RTOL_FP32)}
+    if why:
+        out["failure"] = why
+    for k in ("gpu_over_oracle_rms_error", "last_layer_rms_error_gpu", "last_layer_rms_error_oracle",
+              "last_layer_max_diff_gpu_vs_oracle"):
+        if k in rep:
+            out[k] = rep[k] if isinstance(rep[k], list) else float("%.3g" % rep[k])
+    return out
+
+
+def measure(config, args, torch, frames=None, points_override=None, deep=True, want_parity=True):
+    """Build the pipeline of one configuration, time it, and (deep) take per-layer statistics, eager per-kernel
+    durations and the dominant kernel's roofline position.  frames: list of point arrays timed one after the other
+    in the same buffers (default: the one seeded frame of the preset)."""
+    import numpy as np
+    from sessd3d import api, backbone as B, frames as F
+    preset = dict(PRESETS[config])
+    dtype = args.dtype or preset["dtype"]
+    max_voxels = args.max_voxels or preset["max_voxels"]
+    voxel_cap = args.voxel_cap or preset["voxel_cap"]
+    layers = B.reference_layers(width_mult=preset["width"])
+    W = B.random_weights(layers, seed=1, w_std=0.05 if dtype == "fp16" else 0.1)
+    half = dtype == "fp16"
+    if half:       # FP16 configurations store weights in half: the library and the oracle get the rounded values
+        W = B.Weights([w.astype(np.float16).astype(np.float32) for w in W.w], W.scale, W.shift)
+    if frames is None:
+        frames = [F.lidar_frame(points_override or preset["points"], args.seed, full_circle=preset["full"])]
+    max_points = max(len(f) for f in frames)
+    dev = "cuda:0"
+    kw = dict(feature_dtype=dtype, share_rulebooks=not args.no_share, skip_pad_rows=not args.pad_rows,
+              use_graph=not args.no_graph, overlap_streams=not args.no_overlap, voxel_cap=voxel_cap,
+              dense_size_xyz=B.DENSE_SIZE_XYZ)
+    pipe = api.Pipeline(layers, W, max_points, max_voxels, **kw)
+    points = torch.zeros((max_points, 4), dtype=torch.float32, device=dev)
+    size = torch.zeros((1,), dtype=torch.int32, device=dev)
+    dense = pipe.new_dense(dev)
+    stream = torch.cuda.Stream()
+
+    def upload(pts):
+        buf = np.zeros((max_points, 4), np.float32)
+        buf[:len(pts)] = pts
+        points.copy_(torch.as_tensor(buf))
+        size.copy_(torch.tensor([len(pts)], dtype=torch.int32))
+        torch.cuda.synchronize()
+
+    def timed(steps, warmup):
+        with torch.cuda.stream(stream):
+            for _ in range(warmup):
+                pipe.enqueue(points, size, dense, stream)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        with torch.cuda.stream(stream):
+            for _ in range(steps):
+                pipe.enqueue(points, size, dense, stream)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    per_frame_ms, status = [], 0
+    for i, pts in enumerate(frames):
+        upload(pts)
+        per_frame_ms.append(timed(args.steps, args.warmup if i == 0 else 2))
+        status |= pipe.status(stream)
+    pts = frames[0]
+    if len(frames) > 1:
+        upload(pts)
+        with torch.cuda.stream(stream):
+            pipe.enqueue(points, size, dense, stream)
+        torch.cuda.synchronize()
+    ms_per_frame = float(np.median(per_frame_ms))
+    res = {"config": config, "dtype": dtype, "points": len(pts), "max_voxels": max_voxels, "voxel_cap": voxel_cap,
+           "ms_per_frame": round(ms_per_frame, 4), "status": status, "launches": pipe.num_launches()}
+    if len(frames) > 1:
+        q = np.percentile(per_frame_ms, [10, 50, 90])
+        res["ms_per_frame_p10_p50_p90"] = [round(float(v), 4) for v in q]
+        res["seeded_frames"] = len(frames)
+    res["parity"] = parity_gate(pipe, dense, pts, layers, W, voxel_cap, max_voxels, half) if want_parity else None
+
+    # per-layer active sites / rulebook pairs (small counting kernels, outside the timed region)
+    n_vox, _ = pipe.layer_stats(-1, stream)
+    stats, n_in = [], n_vox
+    for l, layer in enumerate(layers):
+        n_out, pairs = pipe.layer_stats(l, stream)
+        stats.append((n_in, n_out, pairs))
+        n_in = n_out
+    res["voxels"] = n_vox
+
+    # per-kernel durations: HIP events recorded on the pipeline's stream right before and after every launch
+    # (eager launches, one stream).  An event pair that brackets nothing reads a few microseconds on this stream
+    # (`empty_segment`); rocprofv3's kernel trace reads the same few microseconds more than the events minus that
+    # empty time, so the durations used for the roofline are the raw event figures, which agree with the trace.
+    seg, empty = None, 0.0
+    n_prof = args.profile_steps if deep else max(5, args.profile_steps // 5)
+    with torch.cuda.stream(stream):
+        for _ in range(5):
+            pipe.enqueue_timed(points, size, dense, stream)
+        for _ in range(n_prof):
+            s, e = pipe.enqueue_timed(points, size, dense, stream)
+            s = np.asarray(s, np.float64)
+            seg = s if seg is None else seg + s
+            empty += e
+    seg /= n_prof
+    empty /= n_prof
+    esize = 2 if half else 4
+    per_layer = []
+    tot_flops = tot_bytes = 0.0
+    for l, layer in enumerate(layers):
+        n_i, n_o, p = stats[l]
+        fl, by = layer_work(layer, n_i, n_o, p, esize)
+        tot_flops += fl
+        tot_bytes += by
+        g = seg[2 + 2 * l]
+        per_layer.append({"name": layer.name, "n_in": n_i, "n_out": n_o, "pairs": p,
+                          "build_us": round(seg[1 + 2 * l] * 1e3, 2), "gemm_us": round(g * 1e3, 2),
+                          "gemm_tflops": round(fl / (g * 1e-3) / 1e12, 3) if g > 0 else None,
+                          "gemm_gbs": round(by / (g * 1e-3) / 1e9, 1) if g > 0 else None})
+    # dominant kernel: the gather-GEMM instantiation of the widest square layers (64 -> 64, or 128 -> 128)
+    dom_c = 64 * preset["width"]
+    dom = [l for l, layer in enumerate(layers) if layer.cin == dom_c and layer.cout == dom_c]
+    dom_flops = sum(layer_work(layers[l], *stats[l], esize)[0] for l in dom) / len(dom)
+    dom_bytes = sum(layer_work(layers[l], *stats[l], esize)[1] for l in dom) / len(dom)
+    dom_ms = sum(seg[2 + 2 * l] for l in dom) / len(dom)
+    peak_tf = PEAK_FP16_TFLOPS if half else PEAK_FP32_TFLOPS
+    t_mfma = dom_flops / (peak_tf * 1e12)
+    t_hbm = dom_bytes / (PEAK_HBM_GBS * 1e9)
+    if t_mfma >= t_hbm:
+        ach = dom_flops / (dom_ms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": round(ach, 3), "peak": peak_tf, "unit": "TFLOP/s",
+                "frac": round(ach / peak_tf, 4), "traffic": None}
+    else:
+        ach = dom_bytes / (dom_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None}
+    tname = "__half" if half else "float"
+    kname = "conv_mfma<%s, %d, %d, %s>" % (tname, dom_c, dom_c, tname)
+    traffic, fresh = profiled_traffic(kname, config, dtype)
+    roof["traffic"] = traffic
+    roof.update({"traffic_source": "profiles/frame_pipeline_config%d_%s.md (rocprofv3 FETCH_SIZE/WRITE_SIZE), collected on %s"
+                                   % (config, dtype, "this kernel source" if fresh else "an OLDER kernel source: stale"),
+                 "kernel": "gather-GEMM %d->%d (%s)" % (dom_c, dom_c, dtype), "launches_per_frame": len(dom),
+                 "avg_launch_us": round(dom_ms * 1e3, 2),
+                 "avg_launch_us_less_empty_event_pair": round(max(dom_ms - empty, 0.0) * 1e3, 2),
+                 "algorithmic_flops_per_launch": dom_flops, "algorithmic_bytes_per_launch": dom_bytes,
+                 "other_bound_frac": round((dom_bytes / (dom_ms * 1e-3) / 1e9) / PEAK_HBM_GBS, 4) if roof["bound"] == "mfma"
+                 else round((dom_flops / (dom_ms * 1e-3) / 1e12) / peak_tf, 4)})
+    res["roofline"] = roof
+    c_last, dsz = layers[-1].cout, B.DENSE_SIZE_XYZ
+    frame_bytes = 16.0 * len(pts) + 32.0 * n_vox + tot_bytes + stats[-1][1] * (c_last * esize + 16) + \
+        c_last * dsz[0] * dsz[1] * dsz[2] * esize
+    res["frame"] = {"frames_per_s": round(1e3 / ms_per_frame, 1), "algorithmic_gflop": round(tot_flops / 1e9, 3),
+                    "algorithmic_mb": round(frame_bytes / 1e6, 2),
+                    "hbm_roofline_frac": round(frame_bytes / (ms_per_frame * 1e-3) / (PEAK_HBM_GBS * 1e9), 4),
+                    "gemm_launches_sum_us": round(float(sum(seg[2 + 2 * l] for l in range(len(layers)))) * 1e3, 1),
+                    "build_launches_sum_us": round(float(sum(seg[1 + 2 * l] for l in range(len(layers)))) * 1e3, 1),
+                    "eager_segments_ms": {"voxelize": round(seg[0], 4), "sparse2dense": round(seg[-1], 4),
+                                          "sum_raw": round(float(seg.sum()), 4), "empty_segment": round(empty, 5)}}
+    if deep:
+        # latency of single frames (one frame in flight, a synchronise between frames), outside the timed region
+        lat = []
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        for _ in range(min(max(args.steps, 20), 100)):
+            with torch.cuda.stream(stream):
+                ev[0].record(stream)
+                pipe.enqueue(points, size, dense, stream)
+                ev[1].record(stream)
+            stream.synchronize()
+            lat.append(ev[0].elapsed_time(ev[1]))
+        res["frame"]["single_frame_latency_ms_median_p10_p90"] = [round(float(v), 4) for v in np.percentile(lat, [50, 10, 90])]
+        res["layers"] = per_layer
+    else:
+        res["layers"] = [{k: d[k] for k in ("name", "n_out", "pairs", "gemm_us")} for d in per_layer]
+    res["_objects"] = (pts, layers, W, voxel_cap)
+    pipe.close()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=3, choices=[3, 4, 5],
-                    help="benchmark configuration: 3 = 20k points FP32 (headline), 4 = 60k points, voxel cap 40k, FP16, "
-                         "5 = 150k points over 360 degrees, voxel cap 60k, doubled channel widths, FP16")
+                    help="configuration of the headline figure: 3 = 20k points FP32 (default, BASELINE's metric), 4 = 60k points, "
+                         "voxel cap 40k, FP16, 5 = 150k points over 360 degrees, voxel cap 60k, doubled channel widths, FP16")
     ap.add_argument("--points", type=int, default=None)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--dtype", default=None, choices=["fp32", "fp16"])
@@ -113,9 +336,11 @@ def main():
     ap.add_argument("--pad-rows", action="store_true", help="write rows >= voxel_num of every tensor (reference behaviour)")
     ap.add_argument("--no-overlap", action="store_true",
                     help="single stream: do not run the rulebook builds concurrently with the GEMMs of earlier layers")
-    ap.add_argument("--no-two-in-flight", action="store_true",
-                    help="skip the secondary throughput figure (two pipelines on two streams)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-parity", action="store_true", help="skip the comparison with the CPU oracle")
+    ap.add_argument("--no-others", action="store_true", help="only the headline configuration")
+    ap.add_argument("--config5-frames", type=int, default=12,
+                    help="seeded frames of configuration 5 in other_configs (BASELINE names 100; a frame takes ~1 s to generate)")
     ap.add_argument("--profile-steps", type=int, default=50)
     ap.add_argument("--calibrate-mb", type=int, default=0,
                     help="after the timed region run a device-to-device copy of this many MiB three times: a kernel "
@@ -128,170 +353,61 @@ def main():
 
     import numpy as np
     import torch
-    from sessd3d import api, backbone as B, frames as F
+    from sessd3d import frames as F
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
-    dev = "cuda:0"
-    preset = {3: dict(points=20000, dtype="fp32", max_voxels=60000, voxel_cap=60000, width=1, full=False),
-              4: dict(points=60000, dtype="fp16", max_voxels=100000, voxel_cap=40000, width=1, full=False),
-              5: dict(points=150000, dtype="fp16", max_voxels=200000, voxel_cap=60000, width=2, full=True)}[args.config]
-    args.points = args.points or preset["points"]
-    args.dtype = args.dtype or preset["dtype"]
-    args.max_voxels = args.max_voxels or preset["max_voxels"]
-    args.voxel_cap = args.voxel_cap or preset["voxel_cap"]
-    layers = B.reference_layers(width_mult=preset["width"])
-    W = B.random_weights(layers, seed=1, w_std=0.05 if args.dtype == "fp16" else 0.1)
-    pts = F.lidar_frame(args.points, args.seed, full_circle=preset["full"])
-    max_points = args.points
-    pipe = api.Pipeline(layers, W, max_points, args.max_voxels, feature_dtype=args.dtype,
-                        share_rulebooks=not args.no_share, skip_pad_rows=not args.pad_rows,
-                        use_graph=not args.no_graph, overlap_streams=not args.no_overlap, voxel_cap=args.voxel_cap,
-                        dense_size_xyz=B.DENSE_SIZE_XYZ)
-    points = torch.as_tensor(pts).to(dev)
-    size = torch.tensor([len(pts)], dtype=torch.int32, device=dev)
-    dense = pipe.new_dense(dev)
-    stream = torch.cuda.Stream()
-
-    with torch.cuda.stream(stream):
-        for _ in range(args.warmup):
-            pipe.enqueue(points, size, dense, stream)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    with torch.cuda.stream(stream):
-        for _ in range(args.steps):
-            pipe.enqueue(points, size, dense, stream)
-    torch.cuda.synchronize()
-    ms_per_frame = (time.perf_counter() - t0) * 1e3 / args.steps
-    status = pipe.status(stream)
-
-    # latency of single frames (one frame in flight, a synchronise between frames), outside the timed region
-    lat = []
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-    for _ in range(min(args.steps, 100)):
-        with torch.cuda.stream(stream):
-            ev[0].record(stream)
-            pipe.enqueue(points, size, dense, stream)
-            ev[1].record(stream)
-        stream.synchronize()
-        lat.append(ev[0].elapsed_time(ev[1]))
-    lat_q = [round(float(v), 4) for v in np.percentile(lat, [50, 10, 90])]
-
-    # throughput with two frames in flight: a second pipeline on a second stream, frames alternating.  Every
-    # frame does all of its work; only the idle stretches of one frame (its launch-bound head, the narrow
-    # layers) fill with the other's kernels.  Reported beside the headline, never as `value`.
-    two_ms = None
-    if not args.no_two_in_flight:
-        pipe2 = api.Pipeline(layers, W, max_points, args.max_voxels, feature_dtype=args.dtype,
-                             share_rulebooks=not args.no_share, skip_pad_rows=not args.pad_rows,
-                             use_graph=not args.no_graph, overlap_streams=not args.no_overlap,
-                             voxel_cap=args.voxel_cap, dense_size_xyz=B.DENSE_SIZE_XYZ)
-        dense2 = pipe2.new_dense(dev)
-        stream2 = torch.cuda.Stream()
-        lanes = [(pipe, dense, stream), (pipe2, dense2, stream2)]
-
-        def run_pairs(n):
-            for i in range(n):
-                pp, dd, ss = lanes[i & 1]
-                with torch.cuda.stream(ss):
-                    pp.enqueue(points, size, dd, ss)
-
-        run_pairs(2 * max(2, args.warmup // 2))
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        run_pairs(args.steps)
-        torch.cuda.synchronize()
-        two_ms = (time.perf_counter() - t1) * 1e3 / args.steps
-        same = bool(torch.equal(dense, dense2))
-        del pipe2
-
-    # per-layer active sites / rulebook pairs (small counting kernels, outside the timed region)
-    n_vox, _ = pipe.layer_stats(-1, stream)
-    stats, n_in = [], n_vox
-    for l, layer in enumerate(layers):
-        n_out, pairs = pipe.layer_stats(l, stream)
-        stats.append((n_in, n_out, pairs))
-        n_in = n_out
-
-    # per-kernel durations: HIP events on the pipeline's stream around every segment, eager launches
-    # (an event pair that brackets nothing still reads a few microseconds: that empty-segment time is
-    # measured in the same pass and subtracted from every segment)
-    seg, empty = None, 0.0
-    with torch.cuda.stream(stream):
-        for _ in range(5):
-            pipe.enqueue_timed(points, size, dense, stream)
-        for _ in range(args.profile_steps):
-            s, e = pipe.enqueue_timed(points, size, dense, stream)
-            s = np.asarray(s, np.float64)
-            seg = s if seg is None else seg + s
-            empty += e
-    seg /= args.profile_steps
-    empty /= args.profile_steps
-    raw_sum = float(seg.sum())
-    seg = np.maximum(seg - empty, 0.0)
-    esize = 2 if args.dtype == "fp16" else 4
-    per_layer = []
-    tot_flops = tot_bytes = 0.0
-    for l, layer in enumerate(layers):
-        n_i, n_o, p = stats[l]
-        fl, by = layer_work(layer, n_i, n_o, p, esize)
-        tot_flops += fl
-        tot_bytes += by
-        per_layer.append({"name": layer.name, "n_in": n_i, "n_out": n_o, "pairs": p,
-                          "build_us": round(seg[1 + 2 * l] * 1e3, 2), "gemm_us": round(seg[2 + 2 * l] * 1e3, 2),
-                          "gemm_tflops": round(fl / (seg[2 + 2 * l] * 1e-3) / 1e12, 3) if seg[2 + 2 * l] > 0 else None,
-                          "gemm_gbs": round(by / (seg[2 + 2 * l] * 1e-3) / 1e9, 1) if seg[2 + 2 * l] > 0 else None})
-    # dominant kernel: the gather-GEMM instantiation for 64 -> 64 channels (six launches per frame)
-    dom_c = 64 * preset["width"]
-    dom = [l for l, layer in enumerate(layers) if layer.cin == dom_c and layer.cout == dom_c]
-    dom_flops = sum(layer_work(layers[l], *stats[l], esize)[0] for l in dom) / len(dom)
-    dom_bytes = sum(layer_work(layers[l], *stats[l], esize)[1] for l in dom) / len(dom)
-    dom_ms = sum(seg[2 + 2 * l] for l in dom) / len(dom)
-    peak_tf = PEAK_FP16_TFLOPS if args.dtype == "fp16" else PEAK_FP32_TFLOPS
-    t_mfma = dom_flops / (peak_tf * 1e12)
-    t_hbm = dom_bytes / (PEAK_HBM_GBS * 1e9)
-    if t_mfma >= t_hbm:
-        ach = dom_flops / (dom_ms * 1e-3) / 1e12
-        roof = {"bound": "mfma", "achieved": round(ach, 3), "peak": peak_tf, "unit": "TFLOP/s",
-                "frac": round(ach / peak_tf, 4), "traffic": None}
-    else:
-        ach = dom_bytes / (dom_ms * 1e-3) / 1e9
-        roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None}
-    tname = "__half" if args.dtype == "fp16" else "float"
-    kname = "conv_mfma<%s, %d, %d, %s>" % (tname, dom_c, dom_c, tname)
-    roof["traffic"] = profiled_traffic(kname, args.dtype) if args.config == 3 else None
-    roof.update({"kernel": "gather-GEMM %d->%d (%s)" % (dom_c, dom_c, args.dtype), "launches_per_frame": len(dom),
-                 "avg_launch_us": round(dom_ms * 1e3, 2), "algorithmic_flops_per_launch": dom_flops,
-                 "algorithmic_bytes_per_launch": dom_bytes})
-    # whole-frame algorithmic traffic: voxelizer + conv layers + sparse2dense (dense tensor written once)
-    c_last, dsz = layers[-1].cout, B.DENSE_SIZE_XYZ
-    frame_bytes = 16.0 * len(pts) + 32.0 * n_vox + tot_bytes + stats[-1][1] * (c_last * esize + 16) + \
-        c_last * dsz[0] * dsz[1] * dsz[2] * esize
+    want_parity = not args.no_parity
+    head = measure(args.config, args, torch, points_override=args.points, deep=True, want_parity=want_parity)
+    pts, layers, W, voxel_cap = head.pop("_objects")
+    preset = PRESETS[args.config]
     out = {
         "metric": "ms/frame voxelize+3D sparse backbone @~17k voxels",
-        "value": round(ms_per_frame, 4), "unit": "ms/frame", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_frame, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16" if args.dtype == "fp16" else "f32", "data": "synthetic",
+        "value": head["ms_per_frame"], "unit": "ms/frame", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["ms_per_frame"], "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16" if head["dtype"] == "fp16" else "f32", "data": "synthetic",
         "config": {"workload": "config %d: %d-point seeded synthetic LiDAR frame (seed %d), %d voxels, reference 14-layer "
                                "SpMiddleFHD backbone (10 SubM + 4 SparseConv, channel widths x%d, BN folded + ReLU), "
-                               "sparse2Dense to %dx200x176"
-                               % (args.config, len(pts), args.seed, n_vox, preset["width"], layers[-1].cout * 2),
-                   "max_voxels": args.max_voxels, "voxel_cap": args.voxel_cap, "graph": not args.no_graph, "overlap_streams": not args.no_overlap, "share_rulebooks": not args.no_share,
+                               "sparse2Dense to %dx200x176; value = back-to-back graph launches of one frame after the other "
+                               "(single-frame latency: frame.single_frame_latency_ms_median_p10_p90)"
+                               % (args.config, len(pts), args.seed, head["voxels"], preset["width"], layers[-1].cout * 2),
+                   "max_voxels": head["max_voxels"], "voxel_cap": head["voxel_cap"], "graph": not args.no_graph,
+                   "overlap_streams": not args.no_overlap, "share_rulebooks": not args.no_share,
                    "pad_rows": args.pad_rows, "n_layers": len(layers)},
-        "roofline": roof,
-        "frame": {"frames_per_s": round(1e3 / ms_per_frame, 1), "algorithmic_gflop": round(tot_flops / 1e9, 3),
-                  "algorithmic_mb": round(frame_bytes / 1e6, 2),
-                  "hbm_roofline_frac": round(frame_bytes / (ms_per_frame * 1e-3) / (PEAK_HBM_GBS * 1e9), 4),
-                  "single_frame_latency_ms_median_p10_p90": lat_q,
-                  "two_frames_in_flight_ms_per_frame": None if two_ms is None else round(two_ms, 4),
-                  "two_frames_in_flight_outputs_equal": None if two_ms is None else same,
-                  "launches": pipe.num_launches(), "status": status,
-                  "eager_segments_ms": {"voxelize": round(seg[0], 4), "sparse2dense": round(seg[-1], 4),
-                                        "sum_raw": round(raw_sum, 4), "empty_segment": round(empty, 5)}},
-        "layers": per_layer,
+        "roofline": head["roofline"],
+        "parity": head["parity"],
+        "frame": dict(head["frame"], launches=head["launches"], status=head["status"]),
+        "layers": head["layers"],
     }
+    ok = head["status"] == 0 if args.config == 3 else True   # (the voxel cap binds by design in configurations 4 and 5)
+    ok = ok and (head["parity"] is None or head["parity"]["ok"])
+    if not args.no_others:
+        others = []
+        for cfg in (3, 4, 5):
+            if cfg == args.config:
+                continue
+            frames = None
+            if cfg == 5:
+                frames = [F.lidar_frame(PRESETS[5]["points"], 100 + i, full_circle=True) for i in range(max(1, args.config5_frames))]
+            sub = argparse.Namespace(**vars(args))
+            sub.dtype = sub.max_voxels = sub.voxel_cap = None
+            sub.steps, sub.warmup = max(20, min(args.steps, 50)), 5
+            r = measure(cfg, sub, torch, frames=frames, deep=False, want_parity=want_parity)
+            r.pop("_objects")
+            ok = ok and (r["parity"] is None or r["parity"]["ok"])
+            others.append(r)
+        if os.path.exists(KITTI_FRAME0):
+            kitti = np.fromfile(KITTI_FRAME0, np.float32).reshape(-1, 4)
+            sub = argparse.Namespace(**vars(args))
+            sub.dtype = sub.max_voxels = sub.voxel_cap = None
+            sub.steps, sub.warmup = max(20, min(args.steps, 50)), 5
+            r = measure(3, sub, torch, frames=[kitti], deep=False, want_parity=want_parity)
+            r.pop("_objects")
+            r["config"] = "the reference's first frame (KITTI 000000, 20 285 points) through configuration 3's pipeline"
+            ok = ok and (r["parity"] is None or r["parity"]["ok"]) and r["status"] == 0
+            others.append(r)
+        out["other_configs"] = others
     if args.calibrate_mb > 0:
-        src = torch.full((args.calibrate_mb * (1 << 20) // 4,), 1.5, dtype=torch.float32, device=dev)
+        src = torch.full((args.calibrate_mb * (1 << 20) // 4,), 1.5, dtype=torch.float32, device="cuda:0")
         dst = torch.empty_like(src)
         torch.cuda.synchronize()
         for _ in range(3):
@@ -299,8 +415,11 @@ def main():
         torch.cuda.synchronize()
         out["calibration"] = {"copy_mib": args.calibrate_mb, "repeats": 3}
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(pts, layers, W, args.max_voxels, args.voxel_cap)
+        out["cpu_baseline"] = cpu_baseline(pts, layers, W, voxel_cap)
     print(json.dumps(out))
+    if not ok:
+        print("bench.py: parity or status check failed (see \"parity\" / \"status\" in the line above)", file=sys.stderr)
+        sys.exit(1)
 
 
 if __name__ == "__main__":
