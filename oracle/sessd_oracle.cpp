@@ -287,6 +287,13 @@ int oracle_sparse_rulebook(const int32_t* coors, int32_t n, const int32_t* out_s
     int32_t vp[27 * 4];
     for (int32_t v = 0; v < n; ++v) {
         const int32_t c[3] = {coors[v * 4 + 1], coors[v * 4 + 2], coors[v * 4 + 3]};
+        // A negative coordinate: with C's truncating division getValidOutPos then yields kernel offsets outside
+        // [0, K) (e.g. c = -2, k = 3, s = 2, p = 1: o = 0, c - o*s + p = -1) and the reference indexes its rulebook
+        // with them.  Defined here: the row contributes nothing and the status word says so.
+        if (c[0] < 0 || c[1] < 0 || c[2] < 0) {
+            status |= SESSD_STATUS_BAD_COORD;
+            continue;
+        }
         int cnt = oracle_valid_out_pos(c, ksize, stride, padding, dilation, os, vp);
         for (int i = 0; i < cnt; ++i) {
             size_t index = (size_t)vp[i * 4 + 0] * Y * X + (size_t)vp[i * 4 + 1] * X + vp[i * 4 + 2];
@@ -308,6 +315,7 @@ int oracle_sparse_rulebook(const int32_t* coors, int32_t n, const int32_t* out_s
     }
     for (int32_t v = 0; v < n; ++v) {
         const int32_t c[3] = {coors[v * 4 + 1], coors[v * 4 + 2], coors[v * 4 + 3]};
+        if (c[0] < 0 || c[1] < 0 || c[2] < 0) continue;
         int cnt = oracle_valid_out_pos(c, ksize, stride, padding, dilation, os, vp);
         for (int i = 0; i < cnt; ++i) {
             size_t index = (size_t)vp[i * 4 + 0] * Y * X + (size_t)vp[i * 4 + 1] * X + vp[i * 4 + 2];

@@ -19,8 +19,6 @@ LIB = os.path.join(HERE, "lib", "libsessd3d.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-fast-math", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-# experiment hook: extra compiler flags (e.g. -DSESSD_MFMA_WAVES=8) without editing the sources
-FLAGS += os.environ.get("SESSD_EXTRA_FLAGS", "").split()
 
 
 def sources():

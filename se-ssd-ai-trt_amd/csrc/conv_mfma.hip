@@ -42,16 +42,9 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
-#ifndef SESSD_MFMA_WAVES
-#define SESSD_MFMA_WAVES 4
-#endif
-#ifndef SESSD_MFMA_TM
-#define SESSD_MFMA_TM 48
-#endif
-#ifndef SESSD_MFMA_TM_WIDE_F16
-#define SESSD_MFMA_TM_WIDE_F16 64
-#endif
-constexpr int kWaves = SESSD_MFMA_WAVES;
+constexpr int kWaves = 4;           // wave64s per workgroup
+constexpr int kTileRowsBase = 48;   // tile capacity of most kernel instantiations
+constexpr int kTileRowsWideF16 = 64;  // ... and of the wide FP16 ones
 constexpr int kMaxK = kGemmMaxOffsets;
 
 // Tile capacity: most output rows a workgroup can own (<= 64: one wave stages a neighbour list).  The rows
@@ -60,7 +53,7 @@ constexpr int kMaxK = kGemmMaxOffsets;
 // and whose launches are short enough for one tile per CU less to show.  The narrow FP16 layers and
 // Cin = 128 measured slower with 64.
 constexpr int tile_rows(bool half_operands, int cin, int cout) {
-    return half_operands && cin <= 64 && cin * cout >= 32 * 64 ? SESSD_MFMA_TM_WIDE_F16 : SESSD_MFMA_TM;
+    return half_operands && cin <= 64 && cin * cout >= 32 * 64 ? kTileRowsWideF16 : kTileRowsBase;
 }
 
 // Per-dtype shape of one K-chunk: how many channels it spans, what a lane holds of it, and the MFMA

@@ -32,10 +32,7 @@ struct GemmArgs {
 // The target is the tile capacity of the kernel the rulebook's owner runs (gemm_tile_rows()): the tallest
 // tiles the quantisation to whole tiles per CU allows.  Any cut is correct for any kernel: runs longer than
 // a kernel's capacity are walked in pieces.
-#ifndef SESSD_GEMM_MIN_TILE_ROWS
-#define SESSD_GEMM_MIN_TILE_ROWS 48
-#endif
-constexpr int kGemmMinTileRows = SESSD_GEMM_MIN_TILE_ROWS;  // smallest capacity of any kernel: bounds the tile count
+constexpr int kGemmMinTileRows = 48;  // smallest capacity of any kernel: bounds the tile count
 constexpr int kGemmMaxOffsets = 27;  // kernel volumes the rulebook holds (3 x 3 x 3)
 struct TilePlan {
     int count;   // tiles

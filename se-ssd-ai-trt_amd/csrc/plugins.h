@@ -65,9 +65,7 @@ class VoxelGeneratorPlugin {
 // ---------------------------------------------------------------------------------------------
 // Shared by both conv plugins: device weights (+ epilogue), dtype bookkeeping, GEMM dispatch
 // ---------------------------------------------------------------------------------------------
-#ifndef SESSD_TILE_CUT_MIN_WORK
-#define SESSD_TILE_CUT_MIN_WORK (32 * 32)
-#endif
+constexpr int kTileCutMinWork = 32 * 32;  // Cin * Cout from which a rulebook gets equal-work tile cuts
 class ConvPluginBase {
   public:
     virtual ~ConvPluginBase();
@@ -104,7 +102,7 @@ class ConvPluginBase {
     // GEMM runs on the matrix cores and is not tiny
     bool wantTileCuts() const {
         return weights_packed_dev_ != nullptr && !(flags_ & SESSD_FLAG_FORCE_VALU) &&
-               in_channel_ * out_channel_ >= SESSD_TILE_CUT_MIN_WORK;
+               in_channel_ * out_channel_ >= kTileCutMinWork;
     }
     // tile height those cuts aim at: the capacity of this layer's own GEMM kernel
     int tileRows() const;

@@ -73,7 +73,13 @@ sp_insert(const int32_t* __restrict__ coors, const int32_t* __restrict__ voxel_n
     const int c[3] = {cc.y, cc.z, cc.w};
     int o[3], offset;
     uint32_t packed = kEmpty;
-    if (sp_candidate(c, P, e, o, offset)) {
+    // A negative coordinate makes the truncating divisions of getValidOutPos yield kernel offsets outside [0, K)
+    // (c = -2, k = 3, s = 2, p = 1: o = 0, offset term -1), with which the reference indexes its rulebook.  Such a
+    // row contributes nothing here and raises BAD_COORD; the offset is checked as well, so that nothing a caller
+    // passes can make sp_scatter store outside the neighbour table.
+    const bool bad = c[0] < 0 || c[1] < 0 || c[2] < 0;
+    if (bad && e == 0) atomicOr(&meta[0], SESSD_STATUS_BAD_COORD);
+    if (!bad && sp_candidate(c, P, e, o, offset) && offset >= 0 && offset < P.k[0] * P.k[1] * P.k[2]) {
         const uint32_t key = ((uint32_t)o[0] * (uint32_t)P.os[1] + (uint32_t)o[1]) * (uint32_t)P.os[2] + (uint32_t)o[2];
         const int32_t slot = hash_insert(t, key);
         if (slot < 0) {
@@ -184,10 +190,7 @@ struct SparseConv3dLayerPlugin::Layout {
 };
 
 // slots of the candidate hash beyond the worst-case number of distinct candidates: 1/kHashSlack of it
-#ifndef SESSD_SP_HASH_SLACK
-#define SESSD_SP_HASH_SLACK 16
-#endif
-constexpr uint64_t kHashSlack = SESSD_SP_HASH_SLACK;
+constexpr uint64_t kHashSlack = 16;
 
 int SparseConv3dLayerPlugin::maxCandidates() const {
     const int k[3] = {ksize0_, ksize1_, ksize2_}, s[3] = {stride0_, stride1_, stride2_};

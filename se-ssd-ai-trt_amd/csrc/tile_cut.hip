@@ -23,10 +23,7 @@ namespace sessd {
 namespace {
 
 constexpr int kBlock = 256;
-#ifndef SESSD_TILE_ROW_WEIGHT
-#define SESSD_TILE_ROW_WEIGHT 20
-#endif
-constexpr int kRowWeight = SESSD_TILE_ROW_WEIGHT;
+constexpr int kRowWeight = 20;  // fixed cost of a row beside its pairs
 
 __host__ __device__ inline int max_tiles(int max_voxels) { return max_voxels / kGemmMinTileRows + 1024 + 1; }
 

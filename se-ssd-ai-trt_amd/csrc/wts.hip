@@ -11,6 +11,7 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <new>
 #include <memory>
 #include <string>
 #include <vector>
@@ -100,7 +101,17 @@ int sessd_wts_parse(const char* text, size_t length, sessd_wts** out) {
         int64_t size = 0;
         if (!t.next(&b, &e) || !parse_decimal(b, e, &size) || size < 0)
             return fail(SESSD_E_INVALID, "wts: blob '%s' has no valid element count", name.c_str());
-        std::vector<float> v((size_t)size);
+        // every element is a token of at least one character behind a separator: a count the rest of the text cannot
+        // hold is refused before anything of that size is allocated
+        if (size > (int64_t)(t.end - t.p + 1) / 2)
+            return fail(SESSD_E_INVALID, "wts: blob '%s' announces %lld elements, the file ends before that", name.c_str(),
+                        (long long)size);
+        std::vector<float> v;
+        try {
+            v.resize((size_t)size);
+        } catch (const std::bad_alloc&) {
+            return fail(SESSD_E_NOMEM, "wts: blob '%s': no memory for %lld elements", name.c_str(), (long long)size);
+        }
         for (int64_t x = 0; x < size; ++x) {
             uint32_t bits;
             if (!t.next(&b, &e) || !parse_hex32(b, e, &bits))

@@ -476,6 +476,29 @@ def test_sparse_cap_overflow_and_empty():
     assert on == 0 and np.all(out == 0) and np.all(oc == 0) and np.all(num == 0)
 
 
+def test_sparse_layer_refuses_negative_coordinates():
+    """Rows with a negative coordinate (for which getValidOutPos' truncating divisions give kernel offsets outside
+    the rulebook) contribute nothing and raise BAD_COORD; everything else equals the oracle, which drops them too."""
+    layer = SPARSE_LAYERS[0]
+    ig = sparse_input_grid(layer)
+    n, mv = 3000, 16384
+    rng = np.random.default_rng(12)
+    coors = F.clustered_active_voxels(n, (ig[0], 200, 200), 8, n_blobs=30)
+    bad = rng.choice(n, 40, replace=False)
+    coors[bad[:15], 1] = -rng.integers(1, 4, 15)
+    coors[bad[15:30], 2] = -rng.integers(1, 40, 15)
+    coors[bad[30:], 3] = -2
+    feat = rng.uniform(-1, 1, (n, layer.cin)).astype(np.float32)
+    w = rng.normal(0, 0.1, (layer.kvol, layer.cin, layer.cout)).astype(np.float32)
+    conv, out, oc, on, pairs, num = run_sparse(layer, coors, n, feat, w, mv, ig)
+    o_pairs, o_num, o_oc, o_on, o_st = O.sparse_rulebook(coors, n, layer.out_shape, layer.ksize, layer.stride,
+                                                         layer.padding, mv)
+    assert conv.status() == o_st == D.SESSD_STATUS_BAD_COORD
+    assert on == o_on and np.array_equal(oc, o_oc) and np.array_equal(num, o_num)
+    assert not np.isin(pairs[:, 0, :][pairs[:, 0, :] >= 0], bad).any()       # no pair names a refused row
+    assert_features_close(out, O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), RTOL_FP32, "rows with negative coordinates")
+
+
 def test_sparse_generic_stride1_and_corner_truncation():
     """stride 1 (27 candidates per input) and cells at coordinate 0 with padding 0 (C division
     truncates toward zero in getValidOutPos)."""

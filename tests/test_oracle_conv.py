@@ -140,6 +140,33 @@ def test_sparse_rulebook_cap():
     assert got == want
 
 
+def test_kernel_offsets_stay_in_range_for_cells_on_the_grid_and_leave_it_for_negative_ones():
+    """getValidOutPos' offset index lies in [0, K) for every non-negative cell coordinate, over kernel, stride and
+    padding settings that include all of params.h's; a negative coordinate breaks that (C division truncates toward
+    zero), which is why a strided layer refuses such rows (SESSD_STATUS_BAD_COORD) instead of indexing its rulebook
+    with the result, as the reference would."""
+    settings = [((3, 3, 3), (2, 2, 2), (1, 1, 1)), ((3, 3, 3), (2, 2, 2), (0, 1, 1)), ((3, 1, 1), (2, 1, 1), (0, 0, 0)),
+                ((3, 3, 3), (1, 1, 1), (1, 1, 1)), ((2, 2, 2), (2, 2, 2), (0, 0, 0)), ((3, 3, 3), (3, 3, 3), (2, 2, 2)),
+                ((1, 3, 3), (1, 2, 2), (0, 1, 1)), ((3, 3, 3), (2, 2, 2), (2, 2, 2))]
+    for k, s, p in settings:
+        K = k[0] * k[1] * k[2]
+        og = (9, 9, 9)
+        for c in np.ndindex(6, 6, 6):
+            vp = O.valid_out_pos(c, k, s, p, og)
+            assert len(vp) <= 27 and (len(vp) == 0 or (vp[:, 3].min() >= 0 and vp[:, 3].max() < K)), (k, s, p, c)
+    vp = O.valid_out_pos((-2, 0, 0), (3, 3, 3), (2, 2, 2), (1, 1, 1), (9, 9, 9))
+    assert len(vp) and vp[:, 3].min() < 0                       # the reference's arithmetic, restated: out of range
+    # the rulebook builder drops such rows: same result as without them, plus the status bit
+    coors = np.array([[0, 2, 3, 4], [0, -2, 0, 0], [0, 4, 4, 4], [0, 1, -1, 1], [0, 0, 0, 0]], np.int32)
+    good = coors[[0, 2, 4]]
+    args = ((9, 9, 9), (3, 3, 3), (2, 2, 2), (1, 1, 1), 64)
+    pairs, num, oc, on, st = O.sparse_rulebook(coors, len(coors), *args)
+    g_pairs, g_num, g_oc, g_on, g_st = O.sparse_rulebook(good, len(good), *args)
+    assert st == D.SESSD_STATUS_BAD_COORD and g_st == 0
+    assert on == g_on and np.array_equal(oc, g_oc) and np.array_equal(num, g_num)
+    assert np.array_equal(O.canonical_rulebook(pairs, num, coors, oc), O.canonical_rulebook(g_pairs, g_num, good, g_oc))
+
+
 def test_kitti_stage_counts(kitti_frame0):
     with open(GOLDEN) as f:
         gold = json.load(f)

@@ -49,6 +49,8 @@ def test_round_trip_of_the_generator_format(tmp_path):
     ("", "positive blob count"), ("0\n", "positive blob count"), ("x\n", "positive blob count"),
     ("2\na 1 3f800000\n", "2 blobs announced, 1 found"), ("1\na 3 3f800000 3f800000\n", "element 2 of 3"),
     ("1\na 1 3g800000\n", "not 32-bit hex"), ("1\na 1 13f800000\n", "not 32-bit hex"), ("1\na -1\n", "element count"),
+    ("1\na 1000000000000 3f800000\n", "the file ends before that"),       # 2^40 elements announced: refused, not allocated
+    ("1\na 99 3f800000 3f800000\n", "the file ends before that"),
 ])
 def test_malformed_files_are_errors_not_asserts(text, msg):
     with pytest.raises(api.SessdError, match=msg):
