@@ -152,7 +152,7 @@ struct FillRegion {
     uint32_t value;
 };
 struct FillArgs {
-    static constexpr int kMaxRegions = 16;
+    static constexpr int kMaxRegions = 48;
     FillRegion r[kMaxRegions];
     int n = 0;
     bool full() const { return n >= kMaxRegions; }

@@ -139,7 +139,7 @@ struct Pipeline {
             for (size_t l = 0; l < stages.size(); ++l) {
                 auto& st = stages[l];
                 if (!st->ws.p) continue;
-                if (f.n + 5 > FillArgs::kMaxRegions) SESSD_TRY(flush());
+                if (f.n + 6 > FillArgs::kMaxRegions) SESSD_TRY(flush());
                 if (st->subm) st->subm->collectFill(st->ws.p, f, !probes_upstream[l]);
                 else st->sparse->collectFill(st->ws.p, static_cast<int32_t*>(st->coors.p), f);
             }
