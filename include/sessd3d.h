@@ -310,6 +310,47 @@ int sessd_sparse2dense_set_padding(sessd_sparse2dense* h, int32_t top, int32_t b
 void sessd_sparse2dense_destroy(sessd_sparse2dense* h);
 
 /* ------------------------------------------------------------------------------------------ */
+/* Creators by name and clone()  (reference: the four XxxPluginCreator classes and               */
+/* IPluginV2DynamicExt::clone, e.g. submConv3dlayer.cu:732-878, 188-196)                         */
+/* ------------------------------------------------------------------------------------------ */
+/* Values follow nvinfer1::PluginFieldType. */
+enum {
+    SESSD_FIELD_FLOAT16 = 0, SESSD_FIELD_FLOAT32 = 1, SESSD_FIELD_FLOAT64 = 2, SESSD_FIELD_INT8 = 3,
+    SESSD_FIELD_INT16 = 4, SESSD_FIELD_INT32 = 5, SESSD_FIELD_CHAR = 6, SESSD_FIELD_DIMS = 7,
+    SESSD_FIELD_UNKNOWN = 8
+};
+/* Mirrors nvinfer1::PluginField {name, data, type, length} and PluginFieldCollection {nbFields, fields}. */
+typedef struct sessd_plugin_field {
+    const char* name;
+    const void* data;
+    int32_t type;   /* SESSD_FIELD_* */
+    int32_t length; /* elements behind `data` */
+} sessd_plugin_field;
+typedef struct sessd_plugin_field_collection {
+    int32_t nbFields;
+    const sessd_plugin_field* fields;
+} sessd_plugin_field_collection;
+/* replaces XxxPluginCreator::getFieldNames (voxelGenerator.cu:618-647, submConv3dlayer.cu:732-768,
+ * sparseConv3dlayer.cu:918-954, sparse2Dense.cu:316-341): the fields createPlugin reads, `data` NULL,
+ * `length` = the number of elements it reads (0 for weights: the layer shape decides).  plugin_name is the
+ * reference's PLUGIN_NAME: "VoxelGeneratorPlugin", "SubmConv3dLayerPlugin", "SparseConv3dLayerPlugin",
+ * "Sparse2DensePlugin".  NULL for any other name. */
+const sessd_plugin_field_collection* sessd_plugin_field_names(const char* plugin_name);
+/* replaces XxxPluginCreator::createPlugin(name, fc) (voxelGenerator.cu:649-701, submConv3dlayer.cu:770-878,
+ * sparseConv3dlayer.cu:956-1079, sparse2Dense.cu:343-373): fields are picked by name, in any order, unknown
+ * names are ignored; a missing field or a field of the wrong type is an error (the reference builds the
+ * plugin from zeros).  Array fields may carry length 1, as the reference's own creators declare them.
+ * *handle is a sessd_voxelgen* / sessd_submconv3d* / sessd_sparseconv3d* / sessd_sparse2dense*. */
+int sessd_plugin_create(const char* plugin_name, const sessd_plugin_field_collection* fc, void** handle);
+/* replace clone() (voxelGenerator.cu:152-159, submConv3dlayer.cu:188-196, sparseConv3dlayer.cu:204-210,
+ * sparse2Dense.cu:120-125): an independent plugin with its own device copy of the weights, plus what this
+ * library adds to a plugin (epilogue, flags, configured tensor types, dense border). */
+int sessd_voxelgen_clone(const sessd_voxelgen* h, sessd_voxelgen** out);
+int sessd_submconv3d_clone(const sessd_submconv3d* h, sessd_submconv3d** out);
+int sessd_sparseconv3d_clone(const sessd_sparseconv3d* h, sessd_sparseconv3d** out);
+int sessd_sparse2dense_clone(const sessd_sparse2dense* h, sessd_sparse2dense** out);
+
+/* ------------------------------------------------------------------------------------------ */
 /* Frame pipeline: voxelGenerator -> SpMiddleFHD conv stack (+BN+ReLU) -> sparse2Dense          */
 /* (reference wiring: se-ssd-ai-trt.cpp:1138-1252; layer shapes: params.h:19-197)               */
 /* ------------------------------------------------------------------------------------------ */

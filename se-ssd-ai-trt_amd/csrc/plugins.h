@@ -75,6 +75,8 @@ class ConvPluginBase {
                        int nbOutputs);
     // whether this layer's gather-GEMM runs on the MFMA kernel (the one that can take a DenseTarget)
     bool gemmOnMatrixCores() const;
+    // after in_type_ / out_type_ were set by hand (clone): the operand-ordered weight copy for those types
+    int preparePackedForTypes() { return preparePacked(); }
 
     int in_channel_ = 0, out_channel_ = 0, max_voxels_ = 0, feature_num_ = 0;
     int out_shape_x_ = 0, out_shape_y_ = 0, out_shape_z_ = 0;

@@ -102,6 +102,11 @@ def lib():
     L.sessd_pipeline_destroy.argtypes = [vp]
     L.sessd_pipeline_destroy.restype = None
     L.sessd_copy_to_host.argtypes = [vp, vp, sz, vp]
+    L.sessd_plugin_field_names.restype = C.POINTER(D.PluginFieldCollection)
+    L.sessd_plugin_field_names.argtypes = [C.c_char_p]
+    L.sessd_plugin_create.argtypes = [C.c_char_p, C.POINTER(D.PluginFieldCollection), VPP]
+    for name in ("voxelgen", "submconv3d", "sparseconv3d", "sparse2dense"):
+        getattr(L, "sessd_%s_clone" % name).argtypes = [vp, VPP]
     _lib = L
     return L
 
@@ -169,6 +174,15 @@ class _Plugin:
         h = C.c_void_p()
         check(getattr(lib(), "sessd_%s_deserialize" % cls.kind)(blob, len(blob), C.byref(h)))
         obj = cls.__new__(cls)
+        _Plugin.__init__(obj, h)
+        return obj
+
+    def clone(self):
+        """An independent copy (own device weights, same epilogue / flags / configured types): clone() of the reference."""
+        h = C.c_void_p()
+        check(self._fn("clone")(self.h, C.byref(h)))
+        obj = self.__class__.__new__(self.__class__)
+        obj.__dict__.update({k: v for k, v in self.__dict__.items() if k not in ("h", "ws")})
         _Plugin.__init__(obj, h)
         return obj
 
@@ -359,6 +373,49 @@ class Sparse2Dense(_Plugin):
         torch = _torch()
         torch.cuda.synchronize()
         return int(self.ws[:4].view(torch.int32)[0].item())
+
+
+PLUGIN_CLASSES = {}
+
+
+def plugin_field_names(plugin_name):
+    """-> [(name, type, length)] the creator of `plugin_name` reads (getFieldNames of the reference's creators)."""
+    fc = lib().sessd_plugin_field_names(plugin_name.encode())
+    if not fc:
+        raise SessdError(lib().sessd_last_error().decode())
+    return [(fc.contents.fields[i].name.decode(), fc.contents.fields[i].type, fc.contents.fields[i].length)
+            for i in range(fc.contents.nbFields)]
+
+
+def create_plugin(plugin_name, fields):
+    """createPlugin(name, PluginFieldCollection) of the reference's creators: `fields` maps field names to numpy
+    arrays (int32 or float32).  -> the wrapper object of that plugin type."""
+    keep = []
+    arr = (D.PluginField * max(len(fields), 1))()
+    for i, (k, v) in enumerate(fields.items()):
+        a = np.ascontiguousarray(v)
+        keep.append(a)
+        arr[i].name = k.encode()
+        arr[i].data = a.ctypes.data
+        arr[i].type = D.SESSD_FIELD_FLOAT32 if a.dtype == np.float32 else D.SESSD_FIELD_INT32
+        arr[i].length = a.size
+    fc = D.PluginFieldCollection(len(fields), arr)
+    h = C.c_void_p()
+    check(lib().sessd_plugin_create(plugin_name.encode(), C.byref(fc), C.byref(h)))
+    cls = {"VoxelGeneratorPlugin": VoxelGenerator, "SubmConv3dLayerPlugin": SubmConv3d,
+           "SparseConv3dLayerPlugin": SparseConv3d, "Sparse2DensePlugin": Sparse2Dense}[plugin_name]
+    obj = cls.__new__(cls)
+    _Plugin.__init__(obj, h)
+    g = lambda k: np.asarray(fields[k]).reshape(-1)  # noqa: E731
+    if cls is VoxelGenerator:
+        obj.max_voxels = int(g("max_voxels")[0])
+    elif cls is Sparse2Dense:
+        obj.size, obj.channel, obj.padding = tuple(int(v) for v in g("feature_map_size")), int(g("feature_map_channel")[0]), (0, 0, 0, 0)
+    else:
+        obj.max_voxels, obj.cout = int(g("max_voxels")[0]), int(g("out_channel")[0])
+        k = g("ksize")
+        obj.kvol = int(k[0]) ** 3 if cls is SubmConv3d else int(k[0] * k[1] * k[2])
+    return obj
 
 
 def make_conv(layer: B.Layer, weights, prev_grid_xyz, max_voxels, scale=None, shift=None, relu=True):

@@ -69,6 +69,18 @@ class LayerSpec(C.Structure):
                 ("out_shape", C.c_int32 * 3)]
 
 
+SESSD_FIELD_FLOAT32 = 1
+SESSD_FIELD_INT32 = 5
+
+
+class PluginField(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("data", C.c_void_p), ("type", C.c_int32), ("length", C.c_int32)]
+
+
+class PluginFieldCollection(C.Structure):
+    _fields_ = [("nbFields", C.c_int32), ("fields", C.POINTER(PluginField))]
+
+
 FloatPP = C.POINTER(C.POINTER(C.c_float))
 
 

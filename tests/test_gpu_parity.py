@@ -597,3 +597,60 @@ def test_conv_serialization_round_trip():
     assert np.frombuffer(sb[:88], np.int32).tolist() == [64, 64, 60000, 64, 176, 200, 5, 352, 400, 11, 3, 3, 3,
                                                           2, 2, 2, 0, 1, 1, 1, 0, ws.size]
     assert api.SparseConv3d.deserialize(sb).serialize() == sb
+
+
+def test_conv_plugins_by_name_and_their_clones():
+    """createPlugin(name, fields) and clone() of the reference's plugin surface for the two conv plugins: the plugin
+    built from named fields, and its clone (own device weights, epilogue and flags carried over), give the bits of the
+    plugin built from the descriptor."""
+    grid = (21, 200, 176)
+    n, mv = 3000, 4096
+    rng = np.random.default_rng(77)
+    coors = F.clustered_active_voxels(n, grid, 2, n_blobs=30)
+    feat = rng.uniform(-1, 1, (n, 16)).astype(np.float32)
+    w = rng.normal(0, 0.1, (27, 16, 32)).astype(np.float32)
+    sc, sh = rng.uniform(0.5, 1.5, 32).astype(np.float32), rng.uniform(-0.2, 0.2, 32).astype(np.float32)
+    i32 = lambda *v: np.array(v, np.int32)  # noqa: E731
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = np.zeros((mv, 16), np.float32)
+    fbuf[:n] = feat
+    ins = (dev(fbuf), dev(cbuf), dev(np.array([n], np.int32)))
+    # SubM
+    base = api.SubmConv3d(16, 32, grid[::-1], w, mv)
+    named = api.create_plugin("SubmConv3dLayerPlugin", dict(
+        in_channel=i32(16), out_channel=i32(32), max_voxels=i32(mv), feature_num=i32(16), out_shape=i32(*grid[::-1]),
+        spatial_shape=i32(*grid[::-1]), ksize=i32(3), stride=i32(1), padding=i32(1), dilation=i32(1), out_padding=i32(0),
+        weights=w))
+    assert named.serialize() == base.serialize()
+    for p in (base, named):
+        p.set_epilogue(sc, sh, True)
+        p.set_flags(D.SESSD_FLAG_SKIP_PAD_ROWS)
+    twin = named.clone()
+    assert twin.serialize() == named.serialize()
+    named.close()                                         # the clone owns its own copies
+    outs = [to_np(p(*ins))[:n] for p in (base, twin)]
+    torch.cuda.synchronize()
+    assert np.array_equal(outs[0], outs[1]) and np.abs(outs[0]).max() > 0
+    # SparseConv
+    layer = SPARSE_LAYERS[1]
+    ig = sparse_input_grid(layer)
+    coors = F.clustered_active_voxels(n, (ig[0], 200, 176), 4, n_blobs=30)
+    cbuf[:n] = coors
+    feat = rng.uniform(-1, 1, (n, layer.cin)).astype(np.float32)
+    fbuf = np.zeros((mv, layer.cin), np.float32)
+    fbuf[:n] = feat
+    w = rng.normal(0, 0.1, (layer.kvol, layer.cin, layer.cout)).astype(np.float32)
+    ins = (dev(fbuf), dev(cbuf), dev(np.array([n], np.int32)))
+    base = api.SparseConv3d(layer.cin, layer.cout, layer.out_shape, ig[::-1], layer.ksize, layer.stride, layer.padding, w, mv)
+    named = api.create_plugin("SparseConv3dLayerPlugin", dict(
+        in_channel=i32(layer.cin), out_channel=i32(layer.cout), max_voxels=i32(mv), feature_num=i32(layer.cin),
+        out_shape=i32(*layer.out_shape), spatial_shape=i32(*ig[::-1]), ksize=i32(*layer.ksize), stride=i32(*layer.stride),
+        padding=i32(*layer.padding), dilation=i32(1), out_padding=i32(0), weights=w))
+    assert named.serialize() == base.serialize()
+    twin = named.clone()
+    a, b = base(*ins), twin(*ins)
+    torch.cuda.synchronize()
+    na = int(to_np(a[2])[0])
+    assert na == int(to_np(b[2])[0]) > 0 and np.array_equal(to_np(a[1]), to_np(b[1]))
+    assert np.array_equal(to_np(a[0])[:na], to_np(b[0])[:na])

@@ -172,3 +172,49 @@ def test_conv_create_validates_before_touching_the_gpu():
     sd.dilation = 1
     assert L.sessd_sparseconv3d_create(C.byref(sd), w.ctypes.data_as(C.c_void_p), C.byref(h)) == D.SESSD_E_INVALID
     assert L.sessd_submconv3d_create(None, None, None) == D.SESSD_E_INVALID
+
+
+def test_creators_by_name_list_and_read_the_reference_fields():
+    """sessd_plugin_field_names / sessd_plugin_create: the reference's creators by PLUGIN_NAME, fields picked by name."""
+    names = dict((n, [f[0] for f in api.plugin_field_names(n)]) for n in
+                 ("VoxelGeneratorPlugin", "SubmConv3dLayerPlugin", "SparseConv3dLayerPlugin", "Sparse2DensePlugin"))
+    assert names["VoxelGeneratorPlugin"] == ["max_num_points_per_voxel", "max_voxels", "point_cloud_range",
+                                             "voxel_feature_num", "voxel_size"]            # voxelGenerator.cu:624-628
+    conv = ["in_channel", "out_channel", "max_voxels", "feature_num", "out_shape", "spatial_shape", "ksize", "stride",
+            "padding", "dilation", "out_padding", "weights"]                                 # submConv3dlayer.cu:737-748
+    assert names["SubmConv3dLayerPlugin"] == conv and names["SparseConv3dLayerPlugin"] == conv
+    assert names["Sparse2DensePlugin"] == ["feature_map_size", "feature_map_channel"]      # sparse2Dense.cu:321-322
+    assert dict((f[0], f[2]) for f in api.plugin_field_names("SparseConv3dLayerPlugin"))["ksize"] == 3
+    assert dict((f[0], f[2]) for f in api.plugin_field_names("SubmConv3dLayerPlugin"))["ksize"] == 1
+    with pytest.raises(api.SessdError, match="no plugin named"):
+        api.plugin_field_names("ZeroPad2dPlugin")
+    # the voxelizer and sparse2Dense need no GPU to be created: by name == by descriptor, field order free
+    i32, f32 = (lambda *v: np.array(v, np.int32)), (lambda *v: np.array(v, np.float32))
+    vg = api.create_plugin("VoxelGeneratorPlugin", {
+        "voxel_size": f32(*B.VOXEL_SIZE), "max_voxels": i32(20000), "ignored_extra_field": i32(7),
+        "point_cloud_range": f32(*B.POINT_CLOUD_RANGE), "voxel_feature_num": i32(4), "max_num_points_per_voxel": i32(5)})
+    assert vg.serialize() == api.VoxelGenerator(max_voxels=20000).serialize() and vg.grid_size() == (1408, 1600, 40)
+    s2d = api.create_plugin("Sparse2DensePlugin", {"feature_map_channel": i32(64), "feature_map_size": i32(176, 200, 2)})
+    assert s2d.serialize() == api.Sparse2Dense().serialize()
+    with pytest.raises(api.SessdError, match="field 'voxel_size' is missing"):
+        api.create_plugin("VoxelGeneratorPlugin", {"max_voxels": i32(1), "max_num_points_per_voxel": i32(5),
+                                                   "point_cloud_range": f32(*B.POINT_CLOUD_RANGE), "voxel_feature_num": i32(4)})
+    with pytest.raises(api.SessdError, match="has type 5, the creator reads type 1"):
+        api.create_plugin("VoxelGeneratorPlugin", {"max_voxels": i32(1), "max_num_points_per_voxel": i32(5), "voxel_size": i32(1, 1, 1),
+                                                   "point_cloud_range": f32(*B.POINT_CLOUD_RANGE), "voxel_feature_num": i32(4)})
+    with pytest.raises(api.SessdError, match="field 'weights' is missing"):      # checked before any GPU call
+        api.create_plugin("SubmConv3dLayerPlugin", {k: i32(*([3] * (3 if "shape" in k else 1))) for k in conv[:-1]})
+    with pytest.raises(api.SessdError, match="holds 5 values"):
+        api.create_plugin("SubmConv3dLayerPlugin", dict({k: i32(*([3] * (3 if "shape" in k else 1))) for k in conv[:-1]},
+                                                        weights=f32(1, 2, 3, 4, 5)))
+
+
+def test_clone_of_the_gpu_free_plugins():
+    vg = api.VoxelGenerator(max_voxels=1234)
+    vg.set_flags(D.SESSD_FLAG_SKIP_PAD_ROWS)
+    c = vg.clone()
+    assert c.h.value != vg.h.value and c.serialize() == vg.serialize() and c.max_voxels == 1234
+    p = api.Sparse2Dense(padding=(1, 1, 2, 2))
+    c = p.clone()
+    assert c.serialize() == p.serialize() and c.padding == (1, 1, 2, 2)
+    assert api.lib().sessd_voxelgen_clone(None, None) == D.SESSD_E_INVALID
