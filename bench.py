@@ -328,6 +328,9 @@ def main():
                          "voxel cap 40k, FP16, 5 = 150k points over 360 degrees, voxel cap 60k, doubled channel widths, FP16")
     ap.add_argument("--points", type=int, default=None)
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--frame-file", default=None,
+                    help="time this frame file (float32 x,y,z,intensity records, KITTI velodyne layout) instead of the "
+                         "configuration's synthetic frame, e.g. tests/golden/kitti_000000.bin")
     ap.add_argument("--dtype", default=None, choices=["fp32", "fp16"])
     ap.add_argument("--max-voxels", type=int, default=None, help="rows of the conv layers' tensors")
     ap.add_argument("--voxel-cap", type=int, default=None, help="the voxelizer's max_voxels")
@@ -357,7 +360,10 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     want_parity = not args.no_parity
-    head = measure(args.config, args, torch, points_override=args.points, deep=True, want_parity=want_parity)
+    own_frames = None
+    if args.frame_file:
+        own_frames = [np.fromfile(args.frame_file, np.float32).reshape(-1, 4)]
+    head = measure(args.config, args, torch, frames=own_frames, points_override=args.points, deep=True, want_parity=want_parity)
     pts, layers, W, voxel_cap = head.pop("_objects")
     preset = PRESETS[args.config]
     out = {
@@ -365,11 +371,13 @@ def main():
         "value": head["ms_per_frame"], "unit": "ms/frame", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms_per_frame"], "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16" if head["dtype"] == "fp16" else "f32", "data": "synthetic",
-        "config": {"workload": "config %d: %d-point seeded synthetic LiDAR frame (seed %d), %d voxels, reference 14-layer "
+        "config": {"workload": ("frame file %s through " % args.frame_file if args.frame_file else "") +
+                               "config %d: %d-point seeded synthetic LiDAR frame (seed %d), %d voxels, reference 14-layer "
                                "SpMiddleFHD backbone (10 SubM + 4 SparseConv, channel widths x%d, BN folded + ReLU), "
                                "sparse2Dense to %dx200x176; value = back-to-back graph launches of one frame after the other "
                                "(single-frame latency: frame.single_frame_latency_ms_median_p10_p90)"
                                % (args.config, len(pts), args.seed, head["voxels"], preset["width"], layers[-1].cout * 2),
+                   "data_file": args.frame_file,
                    "max_voxels": head["max_voxels"], "voxel_cap": head["voxel_cap"], "graph": not args.no_graph,
                    "overlap_streams": not args.no_overlap, "share_rulebooks": not args.no_share,
                    "pad_rows": args.pad_rows, "n_layers": len(layers)},

@@ -130,6 +130,17 @@ inline HashTable make_hash(uint32_t* keys, uint32_t* vals, uint32_t cap) {
     return t;
 }
 
+// The neighbour table of the SubM layer that comes next on a coors tensor, as the kernel that CREATES the rows
+// of that tensor sees it: it writes "no neighbour" into entries [first_offset, K) of every row it creates, so
+// that the SubM build can run its symmetric lookup (which writes those entries only where a neighbour exists)
+// without the whole K x max_voxels table being cleared per frame.
+struct MirrorInit {
+    int32_t* nbr = nullptr;  // [K][stride]
+    int stride = 0;          // max_voxels of the SubM layer
+    int first_offset = 0;    // 14 for a 3x3x3 kernel: offsets 14..26 are the mirrored ones
+    int K = 0;
+};
+
 // Optional second destination of a gather-GEMM's epilogue: the dense tensor of the sparse2Dense step that
 // would follow (sparse2Dense.cu:182-207: dense[(c*D + z)][y][x] = feat[row][c], here with the zero border of
 // Sparse2DensePlugin::setPadding).  The tensor must already be cleared; its element type is the output

@@ -97,35 +97,47 @@ struct Pipeline {
     int enqueueOverlapped(const void* points, const void* points_size, void* dense, hipStream_t stream) {
         SESSD_HIP_TRY(hipEventRecord(ev_start, stream));
         SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_start, 0));
-        // The voxelizer heads the frame's critical path: it is queued (and, in a graph, submitted) before
-        // anything else.
-        const void* vin[2] = {points, points_size};
-        void* vout[3] = {vg_voxels.p, vg_coors.p, vg_num.p};
-        SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, aux));
-        SESSD_HIP_TRY(hipEventRecord(ev_vg, aux));
         // The kernel that produced a coors tensor has left a cell -> row hash behind (the voxelizer's, or a
         // strided layer's): a SubM layer on the same grid looks its neighbours up in that table and skips its
         // own insert pass (and the clear of its own table).  Keys are (z*Y + y)*X + x: the same number in both
         // grids when X and Y agree; cells of the layer's grid beyond the table's z extent are simply absent.
         // (Beyond 2^20 slots -- 4 MB of keys, one XCD's L2 -- probing the upstream table costs more than the
-        // insert pass it saves.)
-        std::vector<char> probes_upstream(stages.size(), 0);
+        // insert pass it saves.)  The first 3x3x3 SubM rulebook behind a producer is built with the symmetric
+        // lookup (13 probes per row instead of 27): the producer initialises the mirrored entries of the rows
+        // it creates (MirrorInit).
+        std::vector<char> probes_upstream(stages.size(), 0), mirrored(stages.size(), 0);
+        std::vector<MirrorInit> mirror_of(stages.size() + 1);  // [0]: the voxelizer, [l + 1]: strided stage l
         {
             uint32_t mask = vg->cellTable(vg_ws.p, desc.max_points).mask;
             int cx = vg->grid_x_size_, cy = vg->grid_y_size_, cz = vg->grid_z_size_;
+            size_t producer = 0;
             for (size_t l = 0; l < stages.size(); ++l) {
                 ConvStage& st = *stages[l];
                 if (st.subm) {
                     probes_upstream[l] = st.rulebook_from < 0 && st.subm->out_shape_x_ == cx &&
                                          st.subm->out_shape_y_ == cy && st.subm->out_shape_z_ >= cz && mask < (1u << 20);
+                    if (probes_upstream[l] && !mirror_of[producer].nbr) {
+                        const MirrorInit m = st.subm->mirrorInit(st.ws.p);
+                        if (m.nbr) {
+                            mirror_of[producer] = m;
+                            mirrored[l] = 1;
+                        }
+                    }
                 } else {
                     mask = st.sparse->cellTable(st.ws.p).mask;
                     cx = st.sparse->out_shape_x_;
                     cy = st.sparse->out_shape_y_;
                     cz = st.sparse->out_shape_z_;
+                    producer = l + 1;
                 }
             }
         }
+        // The voxelizer heads the frame's critical path: it is queued (and, in a graph, submitted) before
+        // anything else.
+        const void* vin[2] = {points, points_size};
+        void* vout[3] = {vg_voxels.p, vg_coors.p, vg_num.p};
+        SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, aux, mirror_of[0].nbr ? &mirror_of[0] : nullptr));
+        SESSD_HIP_TRY(hipEventRecord(ev_vg, aux));
         SESSD_HIP_TRY(hipStreamWaitEvent(aux_fill, ev_start, 0));
         // every clear of the frame (hash tables, neighbour tables, status words, the dense tensor) has no
         // input: they run batched on a third stream while the voxelizer works
@@ -156,10 +168,12 @@ struct Pipeline {
             ConvStage& st = *stages[l];
             if (st.subm) {
                 if (st.rulebook_from >= 0) continue;
-                SESSD_TRY(st.subm->enqueueBuild(coors, num, st.ws.p, aux, true, probes_upstream[l] ? &cells : nullptr));
+                SESSD_TRY(st.subm->enqueueBuild(coors, num, st.ws.p, aux, true, probes_upstream[l] ? &cells : nullptr,
+                                                mirrored[l] != 0));
             } else {
                 SESSD_TRY(st.sparse->enqueueBuild(coors, num, static_cast<int32_t*>(st.coors.p),
-                                                  static_cast<int32_t*>(st.num.p), st.ws.p, aux, true));
+                                                  static_cast<int32_t*>(st.num.p), st.ws.p, aux, true,
+                                                  mirror_of[l + 1].nbr ? &mirror_of[l + 1] : nullptr));
                 coors = static_cast<const int32_t*>(st.coors.p);
                 num = static_cast<const int32_t*>(st.num.p);
                 cells = st.sparse->cellTable(st.ws.p);

@@ -28,9 +28,10 @@ class VoxelGeneratorPlugin {
                         int nbOutputs);
     size_t getWorkspaceSize(const sessd_tensor_desc* inputs, int nbInputs,
                             const sessd_tensor_desc* outputs, int nbOutputs) const;
+    // `mirror`: the neighbour table of the SubM layer that will run its symmetric lookup on these voxels
     int enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
                 const void* const* inputs, void* const* outputs, void* workspace,
-                hipStream_t stream);
+                hipStream_t stream, const MirrorInit* mirror = nullptr);
     // enqueue() on the library's own static scratch array instead of a caller's workspace: allocates nothing;
     // rejects points tensors whose layout does not fit the array.  Calls that overlap on one GPU race.
     int enqueueStatic(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
@@ -136,8 +137,12 @@ class SubmConv3dLayerPlugin : public ConvPluginBase {
     // enqueue = enqueueBuild (coordinates -> rulebook) + enqueueGemm (features)
     // `cells`: a cell -> row table over this layer's grid that some earlier kernel already built (the
     // voxelizer's, or that of the strided layer that produced `coors`); the insert pass is skipped then
+    // `mirrored`: the producer of `coors` has initialised this layer's mirrored neighbour entries (mirrorInit()):
+    // the lookup then probes 13 offsets per row instead of 27 and writes both directions of every hit
     int enqueueBuild(const int32_t* coors, const int32_t* voxel_num, void* workspace, hipStream_t stream,
-                     bool prefilled = false, const HashTable* cells = nullptr);
+                     bool prefilled = false, const HashTable* cells = nullptr, bool mirrored = false);
+    // what the producer of this layer's coors tensor needs for that (nbr == nullptr: this layer cannot use it)
+    MirrorInit mirrorInit(void* workspace) const;
     void collectFill(void* workspace, FillArgs& f, bool own_table = true) const;
     int enqueueGemm(const void* in_feat, void* out_feat, const int32_t* voxel_num,
                     const void* rulebook_workspace, hipStream_t stream, const DenseTarget* dense = nullptr);
@@ -176,7 +181,7 @@ class SparseConv3dLayerPlugin : public ConvPluginBase {
                        hipStream_t stream) const;
     int countPairs(const void* workspace, uint32_t* indice_num, hipStream_t stream) const;
     int enqueueBuild(const int32_t* coors, const int32_t* voxel_num, int32_t* out_coors, int32_t* out_num,
-                     void* workspace, hipStream_t stream, bool prefilled = false);
+                     void* workspace, hipStream_t stream, bool prefilled = false, const MirrorInit* mirror = nullptr);
     // after enqueueBuild the workspace's hash maps output cell -> output row (see VoxelGeneratorPlugin::cellTable)
     HashTable cellTable(void* workspace) const;
     void collectFill(void* workspace, int32_t* out_coors, FillArgs& f) const;

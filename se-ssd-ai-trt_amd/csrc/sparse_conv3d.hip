@@ -116,7 +116,7 @@ sp_flags(const int32_t* __restrict__ voxel_num, SpParams P, HashTable t, const u
 __global__ void __launch_bounds__(kBlock)
 sp_number(SpParams P, HashTable t, const uint32_t* __restrict__ cand, const uint64_t* __restrict__ first_words,
           const uint32_t* __restrict__ block_counts, int n_blocks, int32_t* __restrict__ out_coors,
-          int32_t* __restrict__ out_num, int32_t* __restrict__ nbr, int K, int32_t* meta) {
+          int32_t* __restrict__ out_num, int32_t* __restrict__ nbr, int K, int32_t* meta, MirrorInit mi) {
     __shared__ uint32_t lds4[4];
     const int b = blockIdx.x;
     const int upto = b == 0 ? n_blocks : b;  // block 0 computes the total
@@ -154,6 +154,9 @@ sp_number(SpParams P, HashTable t, const uint32_t* __restrict__ cand, const uint
     // the new row's neighbour entries start empty (sp_scatter fills in the pairs): clearing them here, row by
     // row, instead of the whole K x max_voxels table before the frame touches only the rows that exist
     for (int k = 0; k < K; ++k) nbr[(size_t)k * P.max_voxels + id] = -1;
+    // ... and so do the mirrored entries of this row in the table of the SubM layer that follows
+    if (mi.nbr && (int)id < mi.stride)
+        for (int k = mi.first_offset; k < mi.K; ++k) mi.nbr[(size_t)k * mi.stride + id] = -1;
 }
 
 __global__ void __launch_bounds__(kBlock)
@@ -368,7 +371,8 @@ void SparseConv3dLayerPlugin::collectFill(void* workspace, int32_t* out_coors, F
 }
 
 int SparseConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* voxel_num, int32_t* out_coors,
-                                          int32_t* out_num, void* workspace, hipStream_t stream, bool prefilled) {
+                                          int32_t* out_num, void* workspace, hipStream_t stream, bool prefilled,
+                                          const MirrorInit* mirror) {
     if (!coors || !voxel_num || !out_coors || !out_num || !workspace)
         return fail(SESSD_E_INVALID, "sparseconv3d.build: null pointer");
     if (reinterpret_cast<uintptr_t>(out_coors) & 15)
@@ -393,7 +397,7 @@ int SparseConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* v
     hipLaunchKernelGGL(sp_insert, grid, block, 0, stream, coors, voxel_num, P, t, L.cand, L.meta);
     hipLaunchKernelGGL(sp_flags, grid, block, 0, stream, voxel_num, P, t, L.cand, L.first_words, L.block_counts);
     hipLaunchKernelGGL(sp_number, grid, block, 0, stream, P, t, L.cand, L.first_words, L.block_counts,
-                       L.n_blocks, out_coors, out_num, L.nbr, kernel_volume_, L.meta);
+                       L.n_blocks, out_coors, out_num, L.nbr, kernel_volume_, L.meta, mirror ? *mirror : MirrorInit());
     hipLaunchKernelGGL(sp_scatter, grid, block, 0, stream, voxel_num, P, t, L.cand, L.nbr);
     SESSD_HIP_TRY(hipGetLastError());
     if (wantTileCuts()) SESSD_TRY(launch_tile_cuts(L.nbr, out_num, kernel_volume_, max_voxels_, tileRows(), L.tiles, stream));

@@ -74,6 +74,35 @@ subm_neighbours(const int32_t* __restrict__ coors, const int32_t* __restrict__ v
     nbr[(size_t)k * max_voxels + v] = res;
 }
 
+// The same lookup for a 3x3x3 kernel over a table whose rows are unique (coordinates made by the voxelizer or a
+// strided layer of this library): the pair (i, o) at offset k is the pair (o, i) at offset 26 - k, so a thread
+// probes only the 13 offsets below the centre and writes both directions of a hit; the centre is the row itself.
+// Entries 14..26 of the active rows must hold -1 before the launch (MirrorInit: the kernel that created the rows
+// wrote them), because only hits are written there.  Half the probes of subm_neighbours.
+__global__ void __launch_bounds__(kBlock)
+subm_neighbours_mirrored(const int32_t* __restrict__ coors, const int32_t* __restrict__ voxel_num, int max_voxels,
+                         Grid3 g, HashTable t, int32_t* __restrict__ nbr, int32_t* meta) {
+    const int v = blockIdx.x * kBlock + threadIdx.x;
+    const int k = blockIdx.y;  // 0 .. 13
+    const int n = clamp_count(voxel_num, max_voxels);
+    if (meta && v == 0 && k == 0) meta[1] = n;
+    if (v >= n) return;
+    if (k == 13) {
+        nbr[(size_t)13 * max_voxels + v] = v;
+        return;
+    }
+    const int4 c = reinterpret_cast<const int4*>(coors)[v];
+    const int z = c.y - 1 + k / 9, y = c.z - 1 + (k / 3) % 3, x = c.w - 1 + k % 3;
+    int32_t res = -1;
+    if (z >= 0 && z < g.Z && y >= 0 && y < g.Y && x >= 0 && x < g.X) {
+        const uint32_t key = ((uint32_t)z * (uint32_t)g.Y + (uint32_t)y) * (uint32_t)g.X + (uint32_t)x;
+        const int32_t slot = hash_find(t, key);
+        if (slot >= 0) res = (int32_t)t.vals[slot];  // (-1 for a cell that was dropped at the capacity)
+    }
+    nbr[(size_t)k * max_voxels + v] = res;
+    if (res >= 0 && res < max_voxels) nbr[(size_t)(26 - k) * max_voxels + res] = v;
+}
+
 }  // namespace
 
 struct SubmConv3dLayerPlugin::Layout {
@@ -234,7 +263,7 @@ void SubmConv3dLayerPlugin::collectFill(void* workspace, FillArgs& f, bool own_t
 }
 
 int SubmConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* voxel_num, void* workspace,
-                                        hipStream_t stream, bool prefilled, const HashTable* cells) {
+                                        hipStream_t stream, bool prefilled, const HashTable* cells, bool mirrored) {
     if (!coors || !voxel_num || !workspace) return fail(SESSD_E_INVALID, "submconv3d.build: null pointer");
     const Layout L = carve(workspace);
     const HashTable t = make_hash(L.keys, L.vals, L.cap);
@@ -248,12 +277,26 @@ int SubmConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* vox
     if (!cells)
         hipLaunchKernelGGL(subm_insert, dim3(row_blocks), dim3(kBlock), 0, stream, coors, voxel_num, max_voxels_,
                            g, t, L.meta);
-    hipLaunchKernelGGL(subm_neighbours, dim3(row_blocks, kernel_volume_), dim3(kBlock), 0, stream, coors,
-                       voxel_num, max_voxels_, g, ksize_, padding_, cells ? *cells : t, L.nbr,
-                       cells ? L.meta : nullptr);
+    if (mirrored && cells && kernel_volume_ == 27)
+        hipLaunchKernelGGL(subm_neighbours_mirrored, dim3(row_blocks, 14), dim3(kBlock), 0, stream, coors, voxel_num,
+                           max_voxels_, g, *cells, L.nbr, L.meta);
+    else
+        hipLaunchKernelGGL(subm_neighbours, dim3(row_blocks, kernel_volume_), dim3(kBlock), 0, stream, coors,
+                           voxel_num, max_voxels_, g, ksize_, padding_, cells ? *cells : t, L.nbr,
+                           cells ? L.meta : nullptr);
     SESSD_HIP_TRY(hipGetLastError());
     if (wantTileCuts()) SESSD_TRY(launch_tile_cuts(L.nbr, voxel_num, kernel_volume_, max_voxels_, tileRows(), L.tiles, stream));
     return SESSD_OK;
+}
+
+MirrorInit SubmConv3dLayerPlugin::mirrorInit(void* workspace) const {
+    MirrorInit m;
+    if (kernel_volume_ != 27 || !workspace) return m;
+    m.nbr = carve(workspace).nbr;
+    m.stride = max_voxels_;
+    m.first_offset = 14;
+    m.K = 27;
+    return m;
 }
 
 int SubmConv3dLayerPlugin::enqueueGemm(const void* in_feat, void* out_feat, const int32_t* voxel_num,

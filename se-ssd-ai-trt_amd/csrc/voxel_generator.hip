@@ -113,7 +113,7 @@ vg_finalize(const float* __restrict__ points, int pf, VgParams p, HashTable t,
             const uint32_t* __restrict__ slots, const int32_t* __restrict__ pt_slot,
             const uint64_t* __restrict__ first_words, const uint32_t* __restrict__ block_counts,
             int n_blocks, float* __restrict__ voxels, int32_t* __restrict__ coors,
-            int32_t* __restrict__ voxel_num, int32_t* status) {
+            int32_t* __restrict__ voxel_num, int32_t* status, MirrorInit mi) {
     __shared__ uint32_t lds4[4];
     const int b = blockIdx.x;
     // block 0 sums every block's count (the total); the others sum the blocks before them
@@ -143,6 +143,8 @@ vg_finalize(const float* __restrict__ points, int pf, VgParams p, HashTable t,
     const int ix = rem - iy * p.gx;
     reinterpret_cast<int4*>(coors)[vid] = make_int4(0, iz, iy, ix);  // voxelGenerator.cu:404-405
     t.vals[slot] = vid;  // the table now maps cell -> voxel row (VoxelGeneratorPlugin::cellTable)
+    if (mi.nbr && (int)vid < mi.stride)  // the next SubM layer's mirrored neighbour entries of this row start empty
+        for (int k = mi.first_offset; k < mi.K; ++k) mi.nbr[(size_t)k * mi.stride + vid] = -1;
 
     // voxelGenerator.cu:274-296: all S slots are summed left to right, unfilled slots count as 0
     const uint32_t* s = slots + (size_t)slot * p.max_pts;
@@ -325,7 +327,7 @@ size_t VoxelGeneratorPlugin::statusOffset(int max_points) const {
 
 int VoxelGeneratorPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc*,
                                   const void* const* inputs, void* const* outputs, void* workspace,
-                                  hipStream_t stream) {
+                                  hipStream_t stream, const MirrorInit* mirror) {
     if (!inputDesc || !inputs || !outputs || !workspace)
         return fail(SESSD_E_INVALID, "voxelgen.enqueue: null argument");
     if (inputDesc[0].nbDims != 3 || inputDesc[0].d[0] != 1)
@@ -367,7 +369,8 @@ int VoxelGeneratorPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sess
     hipLaunchKernelGGL(vg_flags, grid, block, 0, stream, points_size, max_points, pointNum_, L.slots,
                        L.pt_slot, L.first_words, L.block_counts);
     hipLaunchKernelGGL(vg_finalize, grid, block, 0, stream, points, pf, p, t, L.slots, L.pt_slot,
-                       L.first_words, L.block_counts, L.n_blocks, voxels, coors, voxel_num, L.status);
+                       L.first_words, L.block_counts, L.n_blocks, voxels, coors, voxel_num, L.status,
+                       mirror ? *mirror : MirrorInit());
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;
 }
