@@ -35,6 +35,11 @@ extern "C" {
 /* ------------------------------------------------------------------------------------------ */
 
 typedef void* sessd_stream_t; /* a hipStream_t; NULL = the default stream */
+/* For sessd_pipeline_submit only: "the inputs are ready now, order this frame after no stream" (the caller has
+ * synchronised, or the inputs have long been resident).  Without it the frame waits for a marker on the
+ * caller's stream, and where that stream shares a hardware queue with one of the pipeline's own, the marker
+ * sits behind that queue's kernels. */
+#define SESSD_STREAM_NONE ((sessd_stream_t)(intptr_t)-1)
 
 /* Values follow nvinfer1::DataType so descriptors can be copied field by field. */
 enum { SESSD_FLOAT = 0, SESSD_HALF = 1, SESSD_INT32 = 3 };
@@ -391,6 +396,11 @@ typedef struct sessd_pipeline_desc {
     int32_t dense_padding[4];    /* top, bottom, left, right: zero border around the dense tensor
                                     (sessd_sparse2dense_set_padding); the reference network uses 1,1,1,1
                                     (params.h:200-203).  The caller's dense buffer has the padded size */
+    int32_t frames_in_flight;    /* 0 or 1: one frame at a time.  R = 2..8: throughput mode, needs
+                                    overlap_streams.  The pipeline keeps R replicas of its tensors, workspaces and
+                                    graph, each with a stream of its own, and gives successive frames to
+                                    successive replicas, so that frame t + 1 starts while frame t still runs:
+                                    sessd_pipeline_submit / sessd_pipeline_join */
 } sessd_pipeline_desc;
 
 /* Fills `layers[14]` with the reference backbone (params.h:39-192) and `dense`/`voxelgen` with
@@ -436,6 +446,24 @@ int sessd_pipeline_create_from_wts(const sessd_pipeline_desc* desc, const sessd_
 /* points f32[max_points,point_features], points_size i32[1], dense [C*D,H,W]: device pointers */
 int sessd_pipeline_enqueue(sessd_pipeline* h, const void* points, const void* points_size,
                            void* dense, sessd_stream_t stream);
+/* The two halves of sessd_pipeline_enqueue, for hosts that keep several frames in flight (frames_in_flight
+ * >= 2): submit starts the frame once the work already on `stream` is done (the inputs are ready) and
+ * returns a ticket; it does not make `stream` wait for the frame.  join makes `stream` wait until the dense
+ * tensor of that ticket's frame is complete.  Submit frame t + 1 before joining frame t and the two overlap;
+ * enqueue = submit + join.  points, points_size and dense of a frame must stay untouched until its join has
+ * been waited for.  More than frames_in_flight submitted frames without a join in between are safe (a
+ * replica is not reused before its previous frame has finished), they just do not overlap any further.  The
+ * per-layer queries below (layer_io, status, layer_stats, num_launches) then refer to the frame submitted
+ * last.  With frames_in_flight < 2: submit = enqueue, join does nothing. */
+int sessd_pipeline_submit(sessd_pipeline* h, const void* points, const void* points_size, void* dense,
+                          sessd_stream_t stream, int64_t* ticket);
+int sessd_pipeline_join(sessd_pipeline* h, int64_t ticket, sessd_stream_t stream);
+/* join for a host loop: blocks the calling thread (not a stream) until the frame of `ticket` is complete.  A
+ * stream-side join puts a wait into the caller's stream, and where that stream shares a hardware queue with
+ * one of the pipeline's own, everything behind the wait in that queue stands still until the frame is done;
+ * a throughput loop that submits frame t + 1, then waits for frame t + 1 - frames_in_flight here, has no such
+ * coupling.  Only with frames_in_flight >= 2. */
+int sessd_pipeline_wait(sessd_pipeline* h, int64_t ticket);
 /* Device pointers to the tensors a layer produced in the last enqueue (layer = -1: voxelizer).
  * feat: [max_voxels, C]; coors: i32[max_voxels,4]; voxel_num: i32[1]; workspace of that layer. */
 int sessd_pipeline_layer_io(sessd_pipeline* h, int layer, void** feat, void** coors,

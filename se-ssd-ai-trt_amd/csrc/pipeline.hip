@@ -50,6 +50,23 @@ struct ConvStage {
     void* num_ptr = nullptr;
 };
 
+// a captured enqueue sequence, replayed while the pointers it was captured with stay the same
+struct CapturedGraph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    const void* points = nullptr;
+    const void* size = nullptr;
+    void* dense = nullptr;
+    int nodes = -1;
+    void reset() {
+        if (exec) (void)hipGraphExecDestroy(exec);
+        if (graph) (void)hipGraphDestroy(graph);
+        exec = nullptr;
+        graph = nullptr;
+    }
+    ~CapturedGraph() { reset(); }
+};
+
 struct Pipeline {
     sessd_pipeline_desc desc;
     std::unique_ptr<VoxelGeneratorPlugin> vg;
@@ -59,13 +76,17 @@ struct Pipeline {
     sessd_tensor_desc vg_in[2], vg_out[3], s2d_in[3], s2d_out[1];
     int max_voxels = 0;
     size_t device_bytes = 0;
-    // graph replay
-    hipGraph_t graph = nullptr;
-    hipGraphExec_t graph_exec = nullptr;
-    const void* g_points = nullptr;
-    const void* g_size = nullptr;
-    void* g_dense = nullptr;
-    int graph_nodes = -1;
+    CapturedGraph captured;  // graph replay
+
+    // Frames in flight (desc.frames_in_flight = R >= 2): R complete replicas of this pipeline (tensors, workspaces,
+    // graph), used in turn, each on a stream of its own: frame t + 1 starts on the next replica while frame t is
+    // still running on its own, so that the head of one frame and the launch gaps between its kernels fill with the
+    // other frames' work.  `ev_in` / `ev_frame_done` tie a replica's frame to the caller's streams.
+    std::vector<std::unique_ptr<Pipeline>> replicas;
+    hipStream_t frame_stream = nullptr;  // (replica) the stream its frames run on
+    hipEvent_t ev_in = nullptr, ev_frame_done = nullptr;
+    int64_t next_ticket = 0;
+    int last_replica = 0;                       // replica of the last submitted frame (layer_io, status, stats)
 
     // two-stream schedule: coordinate chain (voxelizer + rulebook builds) on `aux`, feature chain on the
     // caller's stream; ev_build[l] = "rulebook of layer l is ready"
@@ -78,8 +99,10 @@ struct Pipeline {
     DeviceBuffer stats;  // u32[32] scratch for per-offset pair counts
 
     ~Pipeline() {
-        if (graph_exec) (void)hipGraphExecDestroy(graph_exec);
-        if (graph) (void)hipGraphDestroy(graph);
+        replicas.clear();
+        for (hipEvent_t e : {ev_in, ev_frame_done})
+            if (e) (void)hipEventDestroy(e);
+        if (frame_stream) (void)hipStreamDestroy(frame_stream);
         for (hipEvent_t e : events) (void)hipEventDestroy(e);
         for (hipEvent_t e : ev_build)
             if (e) (void)hipEventDestroy(e);
@@ -450,55 +473,132 @@ int sessd_reference_backbone(sessd_layer_spec* layers, int max_layers, sessd_vox
 
 int sessd_pipeline_create(const sessd_pipeline_desc* desc, sessd_pipeline** out) {
     if (!desc || !out) return fail(SESSD_E_INVALID, "pipeline_create: null argument");
-    auto* P = new Pipeline();
-    const int rc = build_pipeline(*desc, P);
-    if (rc != SESSD_OK) {
-        delete P;
-        return rc;
+    std::unique_ptr<Pipeline> P(new Pipeline());
+    if (desc->frames_in_flight >= 2) {
+        // R replicas, each a complete pipeline with a stream of its own; this object only holds them and the turn
+        if (desc->frames_in_flight > 8) return fail(SESSD_E_INVALID, "pipeline: at most 8 frames in flight");
+        if (!desc->overlap_streams)
+            return fail(SESSD_E_INVALID, "pipeline: frames_in_flight needs overlap_streams");
+        sessd_pipeline_desc one = *desc;
+        one.frames_in_flight = 0;
+        for (int r = 0; r < desc->frames_in_flight; ++r) {
+            std::unique_ptr<Pipeline> rep(new Pipeline());
+            SESSD_TRY(build_pipeline(one, rep.get()));
+            for (hipEvent_t* e : {&rep->ev_in, &rep->ev_frame_done})
+                SESSD_HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
+            SESSD_HIP_TRY(hipStreamCreateWithFlags(&rep->frame_stream, hipStreamNonBlocking));
+            P->device_bytes += rep->device_bytes;
+            P->max_voxels = rep->max_voxels;
+            P->replicas.push_back(std::move(rep));
+        }
+        P->desc = *desc;
+        P->desc.layers = nullptr;
+        P->desc.weights = P->desc.scale = P->desc.shift = nullptr;
+    } else {
+        SESSD_TRY(build_pipeline(*desc, P.get()));
     }
-    *out = reinterpret_cast<sessd_pipeline*>(P);
+    *out = reinterpret_cast<sessd_pipeline*>(P.release());
     return SESSD_OK;
 }
 
-int sessd_pipeline_enqueue(sessd_pipeline* h, const void* points, const void* points_size, void* dense,
-                           sessd_stream_t stream_) {
-    if (!h || !points || !points_size || !dense) return fail(SESSD_E_INVALID, "pipeline_enqueue: null argument");
+// the pipeline whose tensors a query is about: with frames in flight, the replica of the last submitted frame
+static Pipeline* current(sessd_pipeline* h) {
     auto* P = reinterpret_cast<Pipeline*>(h);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    return P->replicas.empty() ? P : P->replicas[(size_t)P->last_replica].get();
+}
+
+// one frame on `stream`: a replay of the captured graph when the pipeline uses graphs (re-captured when a pointer
+// changed), direct launches otherwise
+static int run_frame(Pipeline* P, const void* points, const void* points_size, void* dense, hipStream_t stream) {
     auto run = [&](hipStream_t st) {
         return P->aux ? P->enqueueOverlapped(points, points_size, dense, st) : P->enqueueDirect(points, points_size, dense, st);
     };
     if (!P->desc.use_graph || stream == nullptr) return run(stream);
-    if (!P->graph_exec || P->g_points != points || P->g_size != points_size || P->g_dense != dense) {
-        if (P->graph_exec) (void)hipGraphExecDestroy(P->graph_exec);
-        if (P->graph) (void)hipGraphDestroy(P->graph);
-        P->graph_exec = nullptr;
-        P->graph = nullptr;
+    CapturedGraph& g = P->captured;
+    if (!g.exec || g.points != points || g.size != points_size || g.dense != dense) {
+        g.reset();
         SESSD_HIP_TRY(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
         const int rc = run(stream);
-        hipGraph_t g = nullptr;
-        const hipError_t e = hipStreamEndCapture(stream, &g);
+        hipGraph_t captured = nullptr;
+        const hipError_t e = hipStreamEndCapture(stream, &captured);
         if (rc != SESSD_OK) {
-            if (g) (void)hipGraphDestroy(g);
+            if (captured) (void)hipGraphDestroy(captured);
             return rc;
         }
         if (e != hipSuccess) return fail(SESSD_E_HIP, "pipeline: stream capture failed: %s", hipGetErrorString(e));
-        P->graph = g;
-        SESSD_HIP_TRY(hipGraphInstantiate(&P->graph_exec, P->graph, nullptr, nullptr, 0));
+        g.graph = captured;
+        SESSD_HIP_TRY(hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0));
         size_t nodes = 0;
-        if (hipGraphGetNodes(P->graph, nullptr, &nodes) == hipSuccess) P->graph_nodes = (int)nodes;
-        P->g_points = points;
-        P->g_size = points_size;
-        P->g_dense = dense;
+        if (hipGraphGetNodes(g.graph, nullptr, &nodes) == hipSuccess) g.nodes = (int)nodes;
+        g.points = points;
+        g.size = points_size;
+        g.dense = dense;
     }
-    SESSD_HIP_TRY(hipGraphLaunch(P->graph_exec, stream));
+    SESSD_HIP_TRY(hipGraphLaunch(g.exec, stream));
     return SESSD_OK;
+}
+
+int sessd_pipeline_submit(sessd_pipeline* h, const void* points, const void* points_size, void* dense,
+                          sessd_stream_t stream_, int64_t* ticket) {
+    if (!h || !points || !points_size || !dense) return fail(SESSD_E_INVALID, "pipeline_submit: null argument");
+    auto* P = reinterpret_cast<Pipeline*>(h);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int64_t t = P->next_ticket;
+    if (P->replicas.empty()) {  // one frame at a time: the frame runs on the caller's stream, join has nothing to add
+        if (stream_ == SESSD_STREAM_NONE) return fail(SESSD_E_INVALID, "pipeline_submit: SESSD_STREAM_NONE needs frames_in_flight >= 2");
+        SESSD_TRY(run_frame(P, points, points_size, dense, stream));
+    } else {
+        const int r = (int)(t % (int64_t)P->replicas.size());
+        Pipeline* R = P->replicas[(size_t)r].get();
+        // the frame starts on the replica's own stream once the caller's inputs are ready (the replica's previous
+        // frame precedes it on that stream)
+        if (stream_ != SESSD_STREAM_NONE) {
+            SESSD_HIP_TRY(hipEventRecord(R->ev_in, stream));
+            SESSD_HIP_TRY(hipStreamWaitEvent(R->frame_stream, R->ev_in, 0));
+        }
+        SESSD_TRY(run_frame(R, points, points_size, dense, R->frame_stream));
+        SESSD_HIP_TRY(hipEventRecord(R->ev_frame_done, R->frame_stream));
+        P->last_replica = r;
+    }
+    P->next_ticket = t + 1;
+    if (ticket) *ticket = t;
+    return SESSD_OK;
+}
+
+int sessd_pipeline_join(sessd_pipeline* h, int64_t ticket, sessd_stream_t stream_) {
+    if (!h) return fail(SESSD_E_INVALID, "pipeline_join: null handle");
+    auto* P = reinterpret_cast<Pipeline*>(h);
+    if (ticket < 0 || ticket >= P->next_ticket) return fail(SESSD_E_INVALID, "pipeline_join: no frame with ticket %lld", (long long)ticket);
+    if (P->replicas.empty()) return SESSD_OK;  // the frame ran on the stream it was submitted on
+    const int64_t R = (int64_t)P->replicas.size();
+    // (a ticket older than the last R frames: its replica has been reused since; waiting for the later frame on
+    // it is at least as strong)
+    Pipeline* rep = P->replicas[(size_t)(ticket % R)].get();
+    SESSD_HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(stream_), rep->ev_frame_done, 0));
+    return SESSD_OK;
+}
+
+int sessd_pipeline_wait(sessd_pipeline* h, int64_t ticket) {
+    if (!h) return fail(SESSD_E_INVALID, "pipeline_wait: null handle");
+    auto* P = reinterpret_cast<Pipeline*>(h);
+    if (ticket < 0 || ticket >= P->next_ticket) return fail(SESSD_E_INVALID, "pipeline_wait: no frame with ticket %lld", (long long)ticket);
+    if (P->replicas.empty()) return fail(SESSD_E_INVALID, "pipeline_wait: this pipeline runs its frames on the caller's stream; synchronise that");
+    Pipeline* rep = P->replicas[(size_t)(ticket % (int64_t)P->replicas.size())].get();
+    SESSD_HIP_TRY(hipEventSynchronize(rep->ev_frame_done));
+    return SESSD_OK;
+}
+
+int sessd_pipeline_enqueue(sessd_pipeline* h, const void* points, const void* points_size, void* dense,
+                           sessd_stream_t stream) {
+    int64_t ticket = 0;
+    SESSD_TRY(sessd_pipeline_submit(h, points, points_size, dense, stream, &ticket));
+    return sessd_pipeline_join(h, ticket, stream);
 }
 
 int sessd_pipeline_layer_io(sessd_pipeline* h, int layer, void** feat, void** coors, void** voxel_num,
                             void** workspace, int32_t* channels) {
     if (!h) return fail(SESSD_E_INVALID, "pipeline_layer_io: null handle");
-    auto* P = reinterpret_cast<Pipeline*>(h);
+    Pipeline* P = current(h);
     if (layer < -1 || layer >= (int)P->stages.size()) return fail(SESSD_E_INVALID, "pipeline_layer_io: no layer %d", layer);
     void* f = P->vg_voxels.p;
     void* c = P->vg_coors.p;
@@ -525,7 +625,7 @@ int sessd_pipeline_layer_io(sessd_pipeline* h, int layer, void** feat, void** co
 
 int sessd_pipeline_status(sessd_pipeline* h, sessd_stream_t stream_, int32_t* status) {
     if (!h || !status) return fail(SESSD_E_INVALID, "pipeline_status: null argument");
-    auto* P = reinterpret_cast<Pipeline*>(h);
+    Pipeline* P = current(h);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     int32_t acc = 0, s = 0;
     SESSD_TRY(read_status_word(P->vg_ws.p, P->vg->statusOffset(P->desc.max_points), stream, &s));
@@ -546,7 +646,7 @@ int sessd_pipeline_enqueue_timed(sessd_pipeline* h, const void* points, const vo
                                  sessd_stream_t stream_, float* segment_ms, int max_segments, int* n_segments) {
     if (!h || !points || !points_size || !dense || !segment_ms || !n_segments)
         return fail(SESSD_E_INVALID, "pipeline_enqueue_timed: null argument");
-    auto* P = reinterpret_cast<Pipeline*>(h);
+    Pipeline* P = current(h);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const int L = (int)P->stages.size();
     const int n_seg = 2 * L + 2;  // voxelizer, {rulebook build, gather-GEMM} per layer, sparse2dense
@@ -593,12 +693,12 @@ int sessd_pipeline_enqueue_timed(sessd_pipeline* h, const void* points, const vo
 int sessd_pipeline_layer_stats(sessd_pipeline* h, int layer, sessd_stream_t stream_, int64_t* n_out,
                                int64_t* pairs) {
     if (!h || !n_out || !pairs) return fail(SESSD_E_INVALID, "pipeline_layer_stats: null argument");
-    auto* P = reinterpret_cast<Pipeline*>(h);
+    Pipeline* P = current(h);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (layer < -1 || layer >= (int)P->stages.size()) return fail(SESSD_E_INVALID, "pipeline_layer_stats: no layer %d", layer);
     void* num = nullptr;
     void* ws = nullptr;
-    SESSD_TRY(sessd_pipeline_layer_io(h, layer, nullptr, nullptr, &num, &ws, nullptr));
+    SESSD_TRY(sessd_pipeline_layer_io(h, layer, nullptr, nullptr, &num, &ws, nullptr));  // (of the same replica)
     int32_t n = 0;
     SESSD_HIP_TRY(hipMemcpyAsync(&n, num, sizeof(n), hipMemcpyDeviceToHost, stream));
     SESSD_HIP_TRY(hipStreamSynchronize(stream));
@@ -623,7 +723,10 @@ size_t sessd_pipeline_device_bytes(const sessd_pipeline* h) {
 }
 
 int sessd_pipeline_num_launches(const sessd_pipeline* h) {
-    return h ? reinterpret_cast<const Pipeline*>(h)->graph_nodes : -1;
+    if (!h) return -1;
+    const Pipeline* P = reinterpret_cast<const Pipeline*>(h);
+    if (!P->replicas.empty()) P = P->replicas[(size_t)P->last_replica].get();
+    return P->captured.nodes;
 }
 
 void sessd_pipeline_destroy(sessd_pipeline* h) { delete reinterpret_cast<Pipeline*>(h); }

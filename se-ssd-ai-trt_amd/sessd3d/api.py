@@ -92,6 +92,9 @@ def lib():
                                            C.POINTER(D.Sparse2DenseDesc)]
     L.sessd_pipeline_create.argtypes = [C.POINTER(D.PipelineDesc), VPP]
     L.sessd_pipeline_enqueue.argtypes = [vp, vp, vp, vp, vp]
+    L.sessd_pipeline_submit.argtypes = [vp, vp, vp, vp, vp, C.POINTER(C.c_int64)]
+    L.sessd_pipeline_join.argtypes = [vp, C.c_int64, vp]
+    L.sessd_pipeline_wait.argtypes = [vp, C.c_int64]
     L.sessd_pipeline_layer_io.argtypes = [vp, C.c_int, VPP, VPP, VPP, VPP, C.POINTER(i32)]
     L.sessd_pipeline_status.argtypes = [vp, vp, C.POINTER(i32)]
     L.sessd_pipeline_enqueue_timed.argtypes = [vp, vp, vp, vp, vp, C.POINTER(C.c_float), C.c_int, C.POINTER(C.c_int)]
@@ -119,6 +122,14 @@ def check(rc):
 def _torch():
     import torch
     return torch
+
+
+class _NoStream:
+    """SESSD_STREAM_NONE of the header: Pipeline.submit orders the frame after no stream (the inputs are ready)."""
+    cuda_stream = -1
+
+
+STREAM_NONE = _NoStream()
 
 
 def _stream_ptr(stream=None):
@@ -492,7 +503,7 @@ class Pipeline:
                  feature_dtype="fp32", relu=True, share_rulebooks=True, skip_pad_rows=False, use_graph=False,
                  dense_size_xyz=B.DENSE_SIZE_XYZ, max_pts_per_voxel=B.MAX_NUM_POINTS_PER_VOXEL,
                  use_epilogue=True, overlap_streams=False, voxel_cap=None, dense_padding=(0, 0, 0, 0),
-                 force_valu=False):
+                 force_valu=False, frames_in_flight=0):
         """max_voxels = rows of every conv-layer tensor; voxel_cap (default: max_voxels) = the voxelizer's
         own limit.  force_valu: every gather-GEMM on the shape-agnostic VALU kernel (cross-checks)."""
         torch = _torch()
@@ -529,6 +540,7 @@ class Pipeline:
         d.flags = (D.SESSD_FLAG_SKIP_PAD_ROWS if skip_pad_rows else 0) | (D.SESSD_FLAG_FORCE_VALU if force_valu else 0)
         d.use_graph = int(use_graph)
         d.overlap_streams = int(overlap_streams)
+        d.frames_in_flight = int(frames_in_flight)
         top, bottom, left, right = (int(v) for v in dense_padding)
         d.dense_padding = (C.c_int32 * 4)(top, bottom, left, right)
         self.dense_shape = (c_last * dense_size_xyz[2], dense_size_xyz[1] + top + bottom,
@@ -547,6 +559,21 @@ class Pipeline:
 
     def enqueue(self, points, points_size, dense, stream=None):
         check(lib().sessd_pipeline_enqueue(self.h, _ptr(points), _ptr(points_size), _ptr(dense), _stream_ptr(stream)))
+
+    def submit(self, points, points_size, dense, stream=None):
+        """Start a frame without making `stream` wait for it -> ticket for join() / wait() (sessd_pipeline_submit).
+        stream = STREAM_NONE (frames in flight only): the inputs are ready, the frame waits for nothing."""
+        t = C.c_int64(0)
+        check(lib().sessd_pipeline_submit(self.h, _ptr(points), _ptr(points_size), _ptr(dense), _stream_ptr(stream), C.byref(t)))
+        return t.value
+
+    def join(self, ticket, stream=None):
+        """Make `stream` wait until the frame of `ticket` is complete (sessd_pipeline_join)."""
+        check(lib().sessd_pipeline_join(self.h, ticket, _stream_ptr(stream)))
+
+    def wait(self, ticket):
+        """Block the calling thread until the frame of `ticket` is complete (sessd_pipeline_wait)."""
+        check(lib().sessd_pipeline_wait(self.h, ticket))
 
     def layer_io(self, layer):
         """-> (feat ptr, coors ptr, voxel_num ptr, workspace ptr, channels) of layer (or -1 = voxelizer)"""

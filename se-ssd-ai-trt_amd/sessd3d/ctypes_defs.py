@@ -91,4 +91,4 @@ class PipelineDesc(C.Structure):
                 ("shift", FloatPP), ("relu", C.c_int32), ("feature_dtype", C.c_int32),
                 ("dense", Sparse2DenseDesc), ("share_rulebooks", C.c_int32), ("flags", C.c_int32),
                 ("use_graph", C.c_int32), ("layer_max_voxels", C.c_int32), ("overlap_streams", C.c_int32),
-                ("dense_padding", C.c_int32 * 4)]
+                ("dense_padding", C.c_int32 * 4), ("frames_in_flight", C.c_int32)]

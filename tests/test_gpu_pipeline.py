@@ -304,3 +304,78 @@ def test_stress_configuration_properties():
     back = first.reshape(128, 2, 200, 176)[:, coors[:, 1], coors[:, 2], coors[:, 3]].T
     assert np.array_equal(back.astype(np.float32), feat)
     assert np.isfinite(first.astype(np.float32)).all()
+
+
+def test_frames_in_flight_give_the_bits_of_one_frame_at_a_time():
+    """frames_in_flight = 3: three replicas of the pipeline, successive frames on successive replicas (submit / join).
+    A sequence of DIFFERENT frames, submitted ahead of their joins, must give exactly the dense tensors, statuses and
+    layer counts of the one-frame-at-a-time pipeline; enqueue() on the same object is submit + join."""
+    layers = B.reference_layers()
+    W = B.random_weights(layers, seed=8, w_std=0.05)
+    mp, mv, R = 8192, 16384, 3
+    kw = dict(share_rulebooks=True, skip_pad_rows=True, use_graph=True, overlap_streams=True)
+    one = api.Pipeline(layers, W, mp, mv, **kw)
+    many = api.Pipeline(layers, W, mp, mv, frames_in_flight=R, **kw)
+    frames = [F.lidar_frame(npts, 40 + i) for i, npts in enumerate((6000, 2500, 8000, 50, 7000, 3000, 6500))]
+    stream = torch.cuda.Stream()
+    want, counts = [], []
+    p, n = points_input(frames[0], mp)
+    dense = one.new_dense()
+    for pts in frames:
+        hp, hn = points_input(pts, mp)
+        with torch.cuda.stream(stream):
+            p.copy_(hp)
+            n.copy_(hn)
+            one.enqueue(p, n, dense, stream)
+        stream.synchronize()
+        want.append(to_np(dense).copy())
+        counts.append([one.layer_count(l) for l in range(-1, len(layers))])
+    # every frame in flight has its own input and output buffers (they must stay untouched until its join)
+    ins = [points_input(pts, mp) for pts in frames]
+    outs = [many.new_dense() for _ in frames]
+    tickets = []
+    with torch.cuda.stream(stream):
+        for i in range(len(frames)):
+            tickets.append(many.submit(ins[i][0], ins[i][1], outs[i], stream))
+            if i >= R - 1:
+                many.join(tickets[i - (R - 1)], stream)
+        for t in tickets[-(R - 1):]:
+            many.join(t, stream)
+    stream.synchronize()
+    assert tickets == list(range(len(frames)))
+    for i in range(len(frames)):
+        assert np.array_equal(to_np(outs[i]), want[i]), "frame %d differs with frames in flight" % i
+    assert [many.layer_count(l) for l in range(-1, len(layers))] == counts[-1]        # queries: the frame submitted last
+    assert many.status() == one.status() == 0 and many.num_launches() == one.num_launches()
+    # enqueue = submit + join, again and again into the same buffers
+    for rep in range(4):
+        outs[0].fill_(3.0)
+        with torch.cuda.stream(stream):
+            many.enqueue(ins[2][0], ins[2][1], outs[0], stream)
+        stream.synchronize()
+        assert np.array_equal(to_np(outs[0]), want[2]), rep
+    # host-driven loop: the inputs are resident (synchronised above), nothing is ordered after a stream, the host
+    # blocks on the oldest frame in flight
+    for o in outs:
+        o.fill_(5.0)
+    torch.cuda.synchronize()
+    tickets = []
+    for i in range(len(frames)):
+        tickets.append(many.submit(ins[i][0], ins[i][1], outs[i], api.STREAM_NONE))
+        if i >= R - 1:
+            many.wait(tickets[i - (R - 1)])
+            j = i - (R - 1)
+            assert np.array_equal(to_np(outs[j]), want[j]), "frame %d differs after a host-side wait" % j
+    for t in tickets[-(R - 1):]:
+        many.wait(t)
+    for i in range(len(frames)):
+        assert np.array_equal(to_np(outs[i]), want[i]), i
+    with pytest.raises(api.SessdError, match="no frame with ticket"):
+        many.join(10 ** 6, stream)
+    with pytest.raises(api.SessdError, match="no frame with ticket"):
+        many.wait(10 ** 6)
+    with pytest.raises(api.SessdError, match="STREAM_NONE needs frames_in_flight"):
+        one.submit(p, n, dense, api.STREAM_NONE)
+    with pytest.raises(api.SessdError, match="runs its frames on the caller's stream"):
+        one.wait(one.submit(p, n, dense, stream))
+    stream.synchronize()

@@ -218,3 +218,18 @@ def test_clone_of_the_gpu_free_plugins():
     c = p.clone()
     assert c.serialize() == p.serialize() and c.padding == (1, 1, 2, 2)
     assert api.lib().sessd_voxelgen_clone(None, None) == D.SESSD_E_INVALID
+
+
+def test_pipeline_frames_in_flight_is_validated_before_anything_is_built():
+    L = api.lib()
+    specs = (D.LayerSpec * 14)()
+    d = D.PipelineDesc()
+    assert L.sessd_reference_backbone(specs, 14, C.byref(d.voxelgen), C.byref(d.dense)) == 14
+    d.max_points, d.point_features, d.n_layers, d.layers = 1000, 4, 14, specs
+    h = C.c_void_p()
+    d.frames_in_flight, d.overlap_streams = 9, 1
+    assert L.sessd_pipeline_create(C.byref(d), C.byref(h)) == D.SESSD_E_INVALID and b"at most 8" in L.sessd_last_error()
+    d.frames_in_flight, d.overlap_streams = 3, 0
+    assert L.sessd_pipeline_create(C.byref(d), C.byref(h)) == D.SESSD_E_INVALID and b"overlap_streams" in L.sessd_last_error()
+    assert L.sessd_pipeline_submit(None, None, None, None, None, None) == D.SESSD_E_INVALID
+    assert L.sessd_pipeline_join(None, 0, None) == D.SESSD_E_INVALID
