@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import oracle_lib as O
-from gpu_util import RTOL_END_TO_END, RTOL_FP16, RTOL_FP32, assert_features_close, dev, points_input, to_np
+from gpu_util import RTOL_END_TO_END, RTOL_END_TO_END_FP16, RTOL_FP16, RTOL_FP32, assert_features_close, dev, points_input, to_np
 from sessd3d import api, backbone as B, ctypes_defs as D, frames as F
 
 pytestmark = pytest.mark.gpu
@@ -150,5 +150,5 @@ def test_random_layer_stack_through_the_pipeline(seed):
     assert pipe.status() == ref["status"], what
     assert [pipe.layer_count(l) for l in range(-1, len(layers))] == list(ref["counts"]), what
     assert np.array_equal(pipe.read_layer(len(layers) - 1)[1], ref["coors"]), what
-    assert_features_close(to_np(dense).astype(np.float32), want, 10 * RTOL_FP16 if half else RTOL_END_TO_END, what)
+    assert_features_close(to_np(dense).astype(np.float32), want, RTOL_END_TO_END_FP16 if half else RTOL_END_TO_END, what)
     pipe.close()
