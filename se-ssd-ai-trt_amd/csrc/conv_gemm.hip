@@ -194,7 +194,13 @@ export_pairs(const int32_t* __restrict__ nbr, int max_voxels, int words_per_k,
 
 int launch_mfma(const GemmArgs& a, hipStream_t stream);  // conv_mfma.hip
 
+int launch_tall(const GemmArgs& a, hipStream_t stream);  // conv_tall.hip
+
 int launch_gather_gemm(const GemmArgs& a, hipStream_t stream) {
+    if (!a.force_valu) {  // FP16 3x3x3 layers from 32 channels up: the tall-tile kernel
+        const int rc = launch_tall(a, stream);
+        if (rc != SESSD_E_UNSUPPORTED) return rc;
+    }
     if (!a.force_valu) {
         const int rc = launch_mfma(a, stream);
         if (rc != SESSD_E_UNSUPPORTED) return rc;  // launched (or failed for good)

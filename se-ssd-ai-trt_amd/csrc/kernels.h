@@ -65,6 +65,9 @@ int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_
 // dense target is set but the layer does not run on the MFMA kernel (see gemm_runs_on_mfma)
 int launch_gather_gemm(const GemmArgs& a, hipStream_t stream);
 bool gemm_runs_on_mfma(int K, int cin, int cout, int in_type, int out_type);
+// whether the layer runs on the tall-tile FP16 kernel (conv_tall.hip), which cuts its own tiles: a rulebook whose
+// owner does needs no equal-work cuts
+bool gemm_runs_tall(int K, int cin, int cout, int in_type, int out_type);
 
 // size in bytes of the packed weight copy for this shape/dtype (0 = shape runs on the VALU path)
 size_t packed_weight_bytes(int K, int cin, int cout, int dtype);

@@ -66,6 +66,7 @@ class VoxelGeneratorPlugin {
 // ---------------------------------------------------------------------------------------------
 // Shared by both conv plugins: device weights (+ epilogue), dtype bookkeeping, GEMM dispatch
 // ---------------------------------------------------------------------------------------------
+bool gemm_runs_tall(int K, int cin, int cout, int in_type, int out_type);  // kernels.h
 constexpr int kTileCutMinWork = 32 * 32;  // Cin * Cout from which a rulebook gets equal-work tile cuts
 class ConvPluginBase {
   public:
@@ -105,7 +106,8 @@ class ConvPluginBase {
     // GEMM runs on the matrix cores and is not tiny
     bool wantTileCuts() const {
         return weights_packed_dev_ != nullptr && !(flags_ & SESSD_FLAG_FORCE_VALU) &&
-               in_channel_ * out_channel_ >= kTileCutMinWork;
+               in_channel_ * out_channel_ >= kTileCutMinWork &&
+               !gemm_runs_tall(kernel_volume_, in_channel_, out_channel_, in_type_, out_type_);
     }
     // tile height those cuts aim at: the capacity of this layer's own GEMM kernel
     int tileRows() const;

@@ -654,3 +654,51 @@ def test_conv_plugins_by_name_and_their_clones():
     na = int(to_np(a[2])[0])
     assert na == int(to_np(b[2])[0]) > 0 and np.array_equal(to_np(a[1]), to_np(b[1]))
     assert np.array_equal(to_np(a[0])[:na], to_np(b[0])[:na])
+
+
+# ---------------------------------------------------------------------------------------------
+# the tall-tile FP16 kernel (3x3x3 layers from 32 channels up): tile edges and both tile heights
+# ---------------------------------------------------------------------------------------------
+def _fp16_subm_against_oracle(cin, cout, n, mv, grid, seed, clustered=True, epilogue=True):
+    rng = np.random.default_rng(seed)
+    coors = (F.clustered_active_voxels(n, grid, seed, n_blobs=max(4, n // 100)) if clustered
+             else F.random_active_voxels(n, grid, seed))
+    feat = O.round_to_half(rng.uniform(-1, 1, (n, cin)).astype(np.float32))
+    w = O.round_to_half(rng.normal(0, 0.1, (27, cin, cout)).astype(np.float32))
+    sc = rng.uniform(0.5, 1.5, cout).astype(np.float32) if epilogue else None
+    sh = rng.uniform(-0.2, 0.2, cout).astype(np.float32) if epilogue else None
+    conv = api.SubmConv3d(cin, cout, grid[::-1], w, mv)
+    if epilogue:
+        conv.set_epilogue(sc, sh, True)
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = np.zeros((mv, cin), np.float32)
+    fbuf[:n] = feat
+    out = conv(dev(fbuf, torch.float16), dev(cbuf), dev(np.array([n], np.int32)), out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    o_pairs, o_num, _ = O.subm_rulebook(coors, n, grid[::-1], mv)
+    o_out = O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv)
+    if epilogue:
+        o_out = O.scale_shift_relu(o_out, mv, sc, sh, True)
+    # every row of the tensor: rows >= n are the epilogue of zero (the reference zero-fills, then BN + ReLU)
+    assert_features_close(to_np(out.float()), O.round_to_half(o_out), RTOL_FP16, "tall fp16 %d->%d, %d rows" % (cin, cout, n))
+    conv.close()
+
+
+@pytest.mark.parametrize("cin,cout", [(32, 32), (64, 64), (128, 128)])
+@pytest.mark.parametrize("n", [1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 300])
+def test_tall_fp16_kernel_row_counts_around_its_tiles(cin, cout, n):
+    """A tile of the tall-tile kernel is 64 rows, 16 per wave: row counts on either side of a block, a wave's
+    share and a tile, down to a single row, against the oracle (pad rows included)."""
+    _fp16_subm_against_oracle(cin, cout, n, 512, (5, 40, 40), 900 + n, epilogue=(n % 2 == 1))
+
+
+@pytest.mark.parametrize("cin,cout", [(32, 32), (64, 128), (128, 128)])
+def test_tall_fp16_kernel_with_two_row_blocks_per_wave(cin, cout):
+    """From 2 x 256 x 128 = 65 536 active rows on, a wave owns two 16-row blocks (128-row tiles); 66 000 rows,
+    the last tile partly filled, against the oracle on 16 threads."""
+    O.set_threads(16)
+    try:
+        _fp16_subm_against_oracle(cin, cout, 66000, 66560, (21, 400, 352), 4000 + cin + cout)
+    finally:
+        O.set_threads(1)

@@ -378,3 +378,29 @@ def test_frames_in_flight_give_the_bits_of_one_frame_at_a_time():
     with pytest.raises(api.SessdError, match="runs its frames on the caller's stream"):
         one.wait(one.submit(p, n, dense, stream))
     stream.synchronize()
+
+
+def test_fp16_stack_ending_in_a_3x3x3_layer_scatters_from_the_tall_tile_kernel():
+    """A stack whose LAST layer is a 3x3x3 FP16 layer of 32+ channels: in the overlapped schedule that layer's
+    kernel (the tall-tile one) also writes the dense tensor.  Dense tensor, sites and status against the oracle,
+    and equal to the single-stream schedule's separate scatter bit for bit."""
+    S, P = D.SESSD_LAYER_SUBM, D.SESSD_LAYER_SPARSE
+    layers = [B.Layer("subm0", S, 4, 32, (1408, 1600, 41), (3, 3, 3), (1, 1, 1), (1, 1, 1)),
+              B.Layer("sparse1", P, 32, 64, (704, 800, 21), (3, 3, 3), (2, 2, 2), (1, 1, 1)),
+              B.Layer("sparse2", P, 64, 64, (352, 400, 11), (3, 3, 3), (2, 2, 2), (1, 1, 1)),
+              B.Layer("sparse3", P, 64, 32, (176, 200, 5), (3, 3, 3), (2, 2, 2), (0, 1, 1)),
+              B.Layer("subm4", S, 32, 32, (176, 200, 5), (3, 3, 3), (1, 1, 1), (1, 1, 1))]
+    W = half_weights(B.random_weights(layers, seed=12, w_std=0.08))
+    pts = F.lidar_frame(9000, 33)
+    mv = 16384
+    dsize = (176, 200, 5)
+    kw = dict(feature_dtype="fp16", share_rulebooks=True, skip_pad_rows=True, dense_size_xyz=dsize, dense_padding=(1, 1, 1, 1))
+    fused, d_fused, _ = run_pipeline(pts, layers, W, 9000, mv, use_graph=True, overlap_streams=True, **kw)
+    plain, d_plain, _ = run_pipeline(pts, layers, W, 9000, mv, use_graph=False, overlap_streams=False, **kw)
+    ref = O.frame(pts, B.voxelgen_desc(max_voxels=mv), layers, W, B.dense_desc(dsize, 32), round_half=True)
+    want = np.pad(ref["dense"], ((0, 0), (1, 1), (1, 1)))
+    assert fused.status() == plain.status() == ref["status"] == 0
+    assert [fused.layer_count(l) for l in range(-1, len(layers))] == list(ref["counts"])
+    assert np.array_equal(fused.read_layer(len(layers) - 1)[1], ref["coors"])
+    assert_features_close(to_np(d_fused).astype(np.float32), want, RTOL_END_TO_END_FP16, "dense from the tall-tile kernel")
+    assert torch.equal(d_fused, d_plain)
