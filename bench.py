@@ -47,14 +47,17 @@ def layer_work(layer, n_in, n_out, pairs, esize):
 
 
 def kernel_source_hash():
-    """Short hash of the gather-GEMM kernel's source: the committed counter summaries carry the hash of the source
+    """Short hash of the gather-GEMM kernels' sources: the committed counter summaries carry the hash of the sources
     they were collected on, so a figure taken from them can be told from a stale one."""
-    with open(os.path.join(ROOT, "se-ssd-ai-trt_amd", "csrc", "conv_mfma.hip"), "rb") as f:
-        return hashlib.sha256(f.read()).hexdigest()[:12]
+    h = hashlib.sha256()
+    for name in ("conv_mfma.hip", "conv_tall.hip"):
+        with open(os.path.join(ROOT, "se-ssd-ai-trt_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:12]
 
 
 def profiled_traffic(kernel, config, dtype):
-    """HBM bytes per launch of `kernel` from the committed rocprofv3 summary (FETCH_SIZE and WRITE_SIZE
+    """HBM bytes per launch of the kernel whose name starts with `kernel`, from the committed rocprofv3 summary (FETCH_SIZE and WRITE_SIZE
     runs, scaled by a copy kernel of known size) -> (bytes or None, whether the summary was collected on the
     current kernel source)."""
     path = os.path.join(ROOT, "profiles", "frame_pipeline_config%d_%s.md" % (config, dtype))
@@ -65,7 +68,7 @@ def profiled_traffic(kernel, config, dtype):
                 if line.startswith("kernel source hash"):
                     fresh = kernel_source_hash() in line
                 cells = [c.strip() for c in line.split("|")]
-                if len(cells) >= 8 and cells[1] == kernel and cells[2].isdigit() and value is None:
+                if len(cells) >= 8 and cells[1].startswith(kernel) and cells[2].isdigit() and value is None:
                     value = float(round((float(cells[5]) + float(cells[6])) * 1e6))
     except (OSError, ValueError):
         pass
@@ -306,8 +309,8 @@ def measure(config, args, torch, frames=None, points_override=None, deep=True, w
         ach = dom_bytes / (dom_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None}
-    tname = "__half" if half else "float"
-    kname = "conv_mfma<%s, %d, %d, %s>" % (tname, dom_c, dom_c, tname)
+    # (FP16 3x3x3 layers from 32 channels up run on the tall-tile kernel, everything else on the split-K one)
+    kname = ("conv_tall<%d, %d," if half else "conv_mfma<float, %d, %d,") % (dom_c, dom_c)
     traffic, fresh = profiled_traffic(kname, config, dtype)
     roof["traffic"] = traffic
     roof.update({"traffic_source": "profiles/frame_pipeline_config%d_%s.md (rocprofv3 FETCH_SIZE/WRITE_SIZE), collected on %s"

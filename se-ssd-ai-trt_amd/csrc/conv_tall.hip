@@ -70,7 +70,7 @@ __device__ __forceinline__ float4* weight_slot() {
 template <int CIN, int COUT, int RB, int D, int DW, int KC>
 __device__ __forceinline__ void tall_tile(const __half* __restrict__ in, __half* __restrict__ out,
                                           const void* __restrict__ Wp, const int32_t* __restrict__ nbr, int n,
-                                          int max_voxels, bool has_scale, bool has_shift, int relu,
+                                          int row0, int max_voxels, bool has_scale, bool has_shift, int relu,
                                           DenseTarget dt, int32_t* s_nbr, const float* s_epi) {
     constexpr int G = CIN / 32;        // K-chunks (32 channels) of the inner dimension
     constexpr int NBT = COUT / 16;     // 16-column blocks
@@ -81,7 +81,6 @@ __device__ __forceinline__ void tall_tile(const __half* __restrict__ in, __half*
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int row0 = blockIdx.x * TR;
     if (row0 >= n) return;
 
     // the tile's neighbour lists (rows beyond n: none) -> LDS
@@ -260,14 +259,14 @@ __device__ __forceinline__ void tall_tile(const __half* __restrict__ in, __half*
     }
 }
 
-// RB = 16-row blocks a wave owns when many rows are active (one otherwise: the tile height is chosen on the
-// device from the row count), D = offsets the rows are requested ahead, DW = register sets for weights in flight
+// RB = 16-row blocks a wave owns in a tall tile (one in a short tile: the heights are chosen on the device from
+// the row count), D = offsets the rows are requested ahead, DW = register sets for weights in flight
 template <int CIN, int COUT, int RB, int D, int DW, int KC>
 __global__ void __launch_bounds__(kWaves * 64, 2)
 conv_tall(const __half* __restrict__ in, __half* __restrict__ out, const void* __restrict__ Wp,
           const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels,
           const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad,
-          int rows_for_tall_tiles, DenseTarget dt) {
+          int slots, DenseTarget dt) {
     static_assert(CIN % 32 == 0 && COUT % 16 == 0, "whole MFMA chunks");
     __shared__ int32_t s_nbr[KC * kWaves * RB * 16];
     __shared__ float s_epi[2 * COUT];
@@ -299,11 +298,21 @@ conv_tall(const __half* __restrict__ in, __half* __restrict__ out, const void* _
         s_epi[tid] = scale ? scale[tid] : 1.f;
         s_epi[COUT + tid] = shift ? shift[tid] : 0.f;
     }
-    // tile height: RB blocks per wave when that still leaves two tiles for every compute unit, else one
-    if (RB > 1 && n >= rows_for_tall_tiles)
-        tall_tile<CIN, COUT, RB, D, DW, KC>(in, out, Wp, nbr, n, max_voxels, scale != nullptr, shift != nullptr, relu, dt, s_nbr, s_epi);
+    // Tile heights.  `slots` workgroups are resident at a time.  Up to 64 * slots rows every
+    // tile is 64 rows (one block per wave); beyond that just enough tiles at the head of the grid take RB blocks
+    // per wave for the launch to stay one round of resident workgroups -- a second, mostly empty round costs a
+    // whole tile's time; beyond 64 * RB * slots rows every tile is tall.
+    constexpr int kShort = kWaves * 16, kTall = kShort * RB;
+    int n_tall = 0;
+    if (RB > 1 && n > kShort * slots) {
+        n_tall = (n - kShort * slots + (kTall - kShort) - 1) / (kTall - kShort);
+        if (n_tall > slots) n_tall = (n + kTall - 1) / kTall;
+    }
+    const int b = blockIdx.x;
+    if (b < n_tall)
+        tall_tile<CIN, COUT, RB, D, DW, KC>(in, out, Wp, nbr, n, b * kTall, max_voxels, scale != nullptr, shift != nullptr, relu, dt, s_nbr, s_epi);
     else
-        tall_tile<CIN, COUT, 1, D, DW, KC>(in, out, Wp, nbr, n, max_voxels, scale != nullptr, shift != nullptr, relu, dt, s_nbr, s_epi);
+        tall_tile<CIN, COUT, 1, D, DW, KC>(in, out, Wp, nbr, n, n_tall * kTall + (b - n_tall) * kShort, max_voxels, scale != nullptr, shift != nullptr, relu, dt, s_nbr, s_epi);
 }
 
 template <int CIN, int COUT, int RB, int D, int DW>
@@ -311,12 +320,18 @@ int launch(const GemmArgs& a, hipStream_t stream) {
     if ((size_t)a.max_voxels * CIN * sizeof(__half) >= kOutOfRange) return SESSD_E_UNSUPPORTED;
     const int num_cu = gemm_compute_units();
     const unsigned blocks = (unsigned)((a.max_voxels + 63) / 64);
-    // tall tiles (RB blocks per wave) once they still give every compute unit two workgroups
-    const int rows_for_tall_tiles = 2 * num_cu * kWaves * RB * 16;
+    // workgroups of this instantiation a compute unit holds at a time (registers and LDS decide; asked once)
+    static int per_cu = 0;
+    if (per_cu == 0) {
+        int v = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, conv_tall<CIN, COUT, RB, D, DW, 27>, kWaves * 64, 0) != hipSuccess || v < 1)
+            v = 2;
+        per_cu = v;
+    }
     hipLaunchKernelGGL((conv_tall<CIN, COUT, RB, D, DW, 27>), dim3(blocks), dim3(kWaves * 64), 0, stream,
                        static_cast<const __half*>(a.in_feat), static_cast<__half*>(a.out_feat), a.w_packed, a.nbr,
                        a.num_out, a.max_voxels, a.scale, a.shift, a.relu, a.write_pad_rows,
-                       rows_for_tall_tiles, a.dense);
+                       per_cu * num_cu, a.dense);
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;
 }

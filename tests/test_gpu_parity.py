@@ -693,12 +693,13 @@ def test_tall_fp16_kernel_row_counts_around_its_tiles(cin, cout, n):
     _fp16_subm_against_oracle(cin, cout, n, 512, (5, 40, 40), 900 + n, epilogue=(n % 2 == 1))
 
 
-@pytest.mark.parametrize("cin,cout", [(32, 32), (64, 128), (128, 128)])
-def test_tall_fp16_kernel_with_two_row_blocks_per_wave(cin, cout):
-    """From 2 x 256 x 128 = 65 536 active rows on, a wave owns two 16-row blocks (128-row tiles); 66 000 rows,
-    the last tile partly filled, against the oracle on 16 threads."""
+@pytest.mark.parametrize("cin,cout,n", [(32, 32, 66000), (64, 64, 40000), (64, 128, 66000), (128, 128, 40000), (128, 128, 66000)])
+def test_tall_fp16_kernel_with_two_row_blocks_per_wave(cin, cout, n):
+    """Beyond 64 rows x the workgroups resident at a time, tiles at the head of the grid take two 16-row blocks per
+    wave (128 rows): a launch with short and tall tiles side by side (40 000 rows) and one with tall tiles only
+    (66 000 rows, the last tile partly filled), against the oracle on 16 threads."""
     O.set_threads(16)
     try:
-        _fp16_subm_against_oracle(cin, cout, 66000, 66560, (21, 400, 352), 4000 + cin + cout)
+        _fp16_subm_against_oracle(cin, cout, n, 66560, (21, 400, 352), 4000 + cin + cout)
     finally:
         O.set_threads(1)
