@@ -315,7 +315,7 @@ conv_tall(const __half* __restrict__ in, __half* __restrict__ out, const void* _
         tall_tile<CIN, COUT, 1, D, DW, KC>(in, out, Wp, nbr, n, n_tall * kTall + (b - n_tall) * kShort, max_voxels, scale != nullptr, shift != nullptr, relu, dt, s_nbr, s_epi);
 }
 
-template <int CIN, int COUT, int RB, int D, int DW>
+template <int CIN, int COUT, int RB, int D, int DW, int KC>
 int launch(const GemmArgs& a, hipStream_t stream) {
     if ((size_t)a.max_voxels * CIN * sizeof(__half) >= kOutOfRange) return SESSD_E_UNSUPPORTED;
     const int num_cu = gemm_compute_units();
@@ -324,11 +324,11 @@ int launch(const GemmArgs& a, hipStream_t stream) {
     static int per_cu = 0;
     if (per_cu == 0) {
         int v = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, conv_tall<CIN, COUT, RB, D, DW, 27>, kWaves * 64, 0) != hipSuccess || v < 1)
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, conv_tall<CIN, COUT, RB, D, DW, KC>, kWaves * 64, 0) != hipSuccess || v < 1)
             v = 2;
         per_cu = v;
     }
-    hipLaunchKernelGGL((conv_tall<CIN, COUT, RB, D, DW, 27>), dim3(blocks), dim3(kWaves * 64), 0, stream,
+    hipLaunchKernelGGL((conv_tall<CIN, COUT, RB, D, DW, KC>), dim3(blocks), dim3(kWaves * 64), 0, stream,
                        static_cast<const __half*>(a.in_feat), static_cast<__half*>(a.out_feat), a.w_packed, a.nbr,
                        a.num_out, a.max_voxels, a.scale, a.shift, a.relu, a.write_pad_rows,
                        per_cu * num_cu, a.dense);
@@ -339,20 +339,27 @@ int launch(const GemmArgs& a, hipStream_t stream) {
 }  // namespace
 
 bool gemm_runs_tall(int K, int cin, int cout, int in_type, int out_type) {
-    if (in_type != SESSD_HALF || out_type != SESSD_HALF || K != 27) return false;
+    if (in_type != SESSD_HALF || out_type != SESSD_HALF) return false;
+    if (K == 3) return cin == cout && (cin == 64 || cin == 128);  // the (3,1,1) layer that ends the backbone
+    if (K != 27) return false;
     return (cin == 128 && cout == 128) || (cin == 64 && (cout == 128 || cout == 64)) || (cin == 32 && (cout == 64 || cout == 32));
 }
 
-// FP16 3x3x3 layers whose inner dimension fills whole 32-channel chunks; SESSD_E_UNSUPPORTED otherwise
+// FP16 layers with 3x3x3 (or the reference's last 3x1x1) kernels whose inner dimension fills whole 32-channel chunks;
+// SESSD_E_UNSUPPORTED otherwise
 int launch_tall(const GemmArgs& a, hipStream_t stream) {
     if (!a.w_packed || !gemm_runs_tall(a.K, a.cin, a.cout, a.in_type, a.out_type)) return SESSD_E_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(a.in_feat) | reinterpret_cast<uintptr_t>(a.out_feat)) & 15) return SESSD_E_UNSUPPORTED;
-    // <Cin, Cout, row blocks per wave in tall tiles, offsets the rows are requested ahead, weight register sets>
-    if (a.cin == 128 && a.cout == 128) return launch<128, 128, 2, 2, 1>(a, stream);
-    if (a.cin == 64 && a.cout == 128) return launch<64, 128, 2, 2, 1>(a, stream);
-    if (a.cin == 64 && a.cout == 64) return launch<64, 64, 2, 3, 2>(a, stream);
-    if (a.cin == 32 && a.cout == 64) return launch<32, 64, 2, 3, 2>(a, stream);
-    if (a.cin == 32 && a.cout == 32) return launch<32, 32, 2, 3, 2>(a, stream);
+    // <Cin, Cout, row blocks per wave in tall tiles, offsets the rows are requested ahead, weight register sets, K>
+    if (a.K == 3) {
+        if (a.cin == 128) return launch<128, 128, 2, 2, 1, 3>(a, stream);
+        return launch<64, 64, 2, 2, 2, 3>(a, stream);
+    }
+    if (a.cin == 128 && a.cout == 128) return launch<128, 128, 2, 2, 1, 27>(a, stream);
+    if (a.cin == 64 && a.cout == 128) return launch<64, 128, 2, 2, 1, 27>(a, stream);
+    if (a.cin == 64 && a.cout == 64) return launch<64, 64, 2, 3, 2, 27>(a, stream);
+    if (a.cin == 32 && a.cout == 64) return launch<32, 64, 2, 3, 2, 27>(a, stream);
+    if (a.cin == 32 && a.cout == 32) return launch<32, 32, 2, 3, 2, 27>(a, stream);
     return SESSD_E_UNSUPPORTED;
 }
 
