@@ -33,6 +33,7 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned int v4u32 __attribute__((__vector_size__(16)));
 
 constexpr int kWaves = 4;
+constexpr int kGroupsAhead = 3;  // groups of weight fragments a wave has requested from LDS ahead of the one it multiplies
 constexpr int kMaxK = kGemmMaxOffsets;
 constexpr unsigned kOutOfRange = 0x80000000u;
 constexpr int kRawBuffer = 0x00020000;
@@ -137,11 +138,10 @@ __device__ __forceinline__ void tall_tile(const __half* __restrict__ in, __half*
         }
     };
     // Offset k at position s of the period.  Its weight fragments (one per K-chunk and column block, 16 bytes per
-    // lane) come from LDS in groups of BG, the next group requested before the current one multiplies.  The
-    // offset's other work -- the rows of offset k+D requested, W[k+1] stored to its buffer, W[k+1+DW] requested
-    // -- is dealt over the groups, so that those instructions issue while the matrix cores work on the group
-    // before: issued in one piece ahead of the first MFMA they took as long as the MFMAs themselves (device
-    // timestamps: 600 + 400 of 1900 cycles per offset).
+    // lane) come from LDS in groups of BG, requested kGroupsAhead groups before they multiply.  The offset's other
+    // work -- the rows of offset k+D requested, W[k+1] stored to its buffer, W[k+1+DW] requested -- is dealt over
+    // the groups, so that those instructions issue while the matrix cores work on the group before (issued in one
+    // piece ahead of the first MFMA they took as long as the MFMAs themselves).
     auto offset_step = [&](int k, auto s_c) {
         constexpr int s = decltype(s_c)::value;
         const v4f* const s_w = reinterpret_cast<const v4f*>(weight_slot<U, s % 2>()) + lane;
@@ -150,14 +150,17 @@ __device__ __forceinline__ void tall_tile(const __half* __restrict__ in, __half*
         static_assert(U % BG == 0, "whole groups");
         constexpr int NI = RB + UW;                  // side items: RB row blocks, then UW weight units
         constexpr int IPG = (NI + NG - 1) / NG;      // ... per group
-        v4f b[2][BG];
+        constexpr int PD = NG >= 3 ? kGroupsAhead : 1;  // groups requested ahead
+        v4f b[PD + 1][BG];
 #pragma unroll
-        for (int j = 0; j < BG; ++j) b[0][j] = s_w[j * 64];
+        for (int g0 = 0; g0 < PD; ++g0)
+#pragma unroll
+            for (int j = 0; j < BG; ++j) b[g0][j] = s_w[(g0 * BG + j) * 64];
 #pragma unroll
         for (int grp = 0; grp < NG; ++grp) {
-            if (grp + 1 < NG) {
+            if (grp + PD < NG) {
 #pragma unroll
-                for (int j = 0; j < BG; ++j) b[(grp + 1) & 1][j] = s_w[((grp + 1) * BG + j) * 64];
+                for (int j = 0; j < BG; ++j) b[(grp + PD) % (PD + 1)][j] = s_w[((grp + PD) * BG + j) * 64];
             }
 #pragma unroll
             for (int it = grp * IPG; it < (grp + 1) * IPG && it < NI; ++it) {
@@ -174,7 +177,7 @@ __device__ __forceinline__ void tall_tile(const __half* __restrict__ in, __half*
                 const int f = grp * BG + j, g = f / NBT, nb = f % NBT;
 #pragma unroll
                 for (int blk = 0; blk < RB; ++blk)
-                    acc[blk][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const v8h*>(&b[grp & 1][j]),
+                    acc[blk][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const v8h*>(&b[grp % (PD + 1)][j]),
                                                                          *reinterpret_cast<const v8h*>(&a[s % NBUF][blk][g]),
                                                                          acc[blk][nb], 0, 0, 0);
             }
@@ -352,10 +355,10 @@ int launch_tall(const GemmArgs& a, hipStream_t stream) {
     if ((reinterpret_cast<uintptr_t>(a.in_feat) | reinterpret_cast<uintptr_t>(a.out_feat)) & 15) return SESSD_E_UNSUPPORTED;
     // <Cin, Cout, row blocks per wave in tall tiles, offsets the rows are requested ahead, weight register sets, K>
     if (a.K == 3) {
-        if (a.cin == 128) return launch<128, 128, 2, 2, 1, 3>(a, stream);
+        if (a.cin == 128) return launch<128, 128, 2, 1, 1, 3>(a, stream);
         return launch<64, 64, 2, 2, 2, 3>(a, stream);
     }
-    if (a.cin == 128 && a.cout == 128) return launch<128, 128, 2, 2, 1, 27>(a, stream);
+    if (a.cin == 128 && a.cout == 128) return launch<128, 128, 2, 1, 1, 27>(a, stream);
     if (a.cin == 64 && a.cout == 128) return launch<64, 128, 2, 2, 1, 27>(a, stream);
     if (a.cin == 64 && a.cout == 64) return launch<64, 64, 2, 3, 2, 27>(a, stream);
     if (a.cin == 32 && a.cout == 64) return launch<32, 64, 2, 3, 2, 27>(a, stream);
