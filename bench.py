@@ -268,7 +268,7 @@ def measure(config, args, torch, frames=None, points_override=None, deep=True, w
     # (`empty_segment`); rocprofv3's kernel trace reads the same few microseconds more than the events minus that
     # empty time, so the durations used for the roofline are the raw event figures, which agree with the trace.
     seg, empty = None, 0.0
-    n_prof = args.profile_steps if deep else max(5, args.profile_steps // 5)
+    n_prof = max(1, args.profile_steps) if deep else max(5, args.profile_steps // 5)
     with torch.cuda.stream(stream):
         for _ in range(5):
             pipe.enqueue_timed(points, size, dense, stream)
