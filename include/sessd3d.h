@@ -78,11 +78,7 @@ enum {
     SESSD_FLAG_SKIP_PAD_ROWS = 1,
     /* Run the gather-GEMM on the shape-agnostic VALU kernel even where an MFMA kernel exists
      * (cross-check of the matrix-core path). */
-    SESSD_FLAG_FORCE_VALU = 2,
-    /* FP32 layers: multiply on the FP32 matrix instructions (16x16x4) instead of the default, which splits
-     * every FP32 operand into three BF16 parts and multiplies those (six BF16 matrix instructions per FP32
-     * product, FP32 accumulation; as accurate as an FP32 accumulation, several times faster). */
-    SESSD_FLAG_FP32_MFMA = 4
+    SESSD_FLAG_FORCE_VALU = 2
 };
 
 const char* sessd_last_error(void); /* thread-local text of the last failure */

@@ -11,7 +11,7 @@ int ConvPluginBase::freeDevice() {
     // the reference frees in terminate() and again in the destructor (submConv3dlayer.cu:671-682);
     // here every pointer is released once and cleared
     void** ptrs[] = {reinterpret_cast<void**>(&weights_dev_), reinterpret_cast<void**>(&weights_half_dev_),
-                     &weights_packed_dev_, &weights_split_dev_, reinterpret_cast<void**>(&epi_.scale_dev),
+                     &weights_packed_dev_, reinterpret_cast<void**>(&epi_.scale_dev),
                      reinterpret_cast<void**>(&epi_.shift_dev)};
     for (void** p : ptrs) {
         if (*p) (void)hipFree(*p);
@@ -91,36 +91,23 @@ int ConvPluginBase::preparePacked() {
         SESSD_HIP_TRY(hipMalloc(&weights_packed_dev_, bytes));
         SESSD_HIP_TRY(hipMemcpy(weights_packed_dev_, host.data(), bytes, hipMemcpyHostToDevice));
     }
-    if (weights_split_dev_) (void)hipFree(weights_split_dev_);
-    weights_split_dev_ = nullptr;
-    if (gemm_runs_split(kernel_volume_, in_channel_, out_channel_, in_type_, out_type_)) {
-        const size_t sb = split_weight_bytes(kernel_volume_, in_channel_, out_channel_);
-        std::vector<uint8_t> host(sb);
-        pack_weights_split(weights_data_.data(), kernel_volume_, in_channel_, out_channel_, host.data());
-        SESSD_HIP_TRY(hipMalloc(&weights_split_dev_, sb));
-        SESSD_HIP_TRY(hipMemcpy(weights_split_dev_, host.data(), sb, hipMemcpyHostToDevice));
-    }
     packed_dtype_ = compute_type;
     return SESSD_OK;
 }
 
 bool ConvPluginBase::gemmOnMatrixCores() const {
-    if (gemmOnSplitKernel()) return true;
     return weights_packed_dev_ != nullptr && !(flags_ & SESSD_FLAG_FORCE_VALU) &&
            gemm_runs_on_mfma(kernel_volume_, in_channel_, out_channel_, in_type_, out_type_);
 }
 
 int ConvPluginBase::tileRows() const { return gemm_tile_rows(in_channel_, out_channel_, out_type_); }
 
-GemmArgs ConvPluginBase::gemmArgs(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* tiles,
-                                  const int32_t* num_out, const DenseTarget* dense, const void* in_split,
-                                  void* out_split) const {
+int ConvPluginBase::runGemm(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* tiles,
+                            const int32_t* num_out, hipStream_t stream, const DenseTarget* dense) {
     GemmArgs a;
     if (dense) a.dense = *dense;
     a.in_feat = in_feat;
     a.out_feat = out_feat;
-    a.in_split = in_split;
-    a.out_split = out_split;
     a.nbr = nbr;
     a.num_out = num_out;
     a.max_voxels = max_voxels_;
@@ -132,21 +119,12 @@ GemmArgs ConvPluginBase::gemmArgs(const void* in_feat, void* out_feat, const int
     a.w_f32 = weights_dev_;
     a.w_f16 = weights_half_dev_;
     a.w_packed = weights_packed_dev_;
-    a.w_split = weights_split_dev_;
-    a.fp32_mfma = (flags_ & SESSD_FLAG_FP32_MFMA) ? 1 : 0;
     a.scale = epi_.scale_dev;
     a.shift = epi_.shift_dev;
     a.relu = epi_.relu;
     a.write_pad_rows = (flags_ & SESSD_FLAG_SKIP_PAD_ROWS) ? 0 : 1;
     a.force_valu = (flags_ & SESSD_FLAG_FORCE_VALU) ? 1 : 0;
     a.tiles = tiles;
-    return a;
-}
-
-int ConvPluginBase::runGemm(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* tiles,
-                            const int32_t* num_out, hipStream_t stream, const DenseTarget* dense,
-                            const void* in_split, void* out_split) {
-    const GemmArgs a = gemmArgs(in_feat, out_feat, nbr, tiles, num_out, dense, in_split, out_split);
     if (ev_gemm_begin_) SESSD_HIP_TRY(hipEventRecord(ev_gemm_begin_, stream));
     SESSD_TRY(launch_gather_gemm(a, stream));
     if (ev_gemm_end_) SESSD_HIP_TRY(hipEventRecord(ev_gemm_end_, stream));

@@ -196,22 +196,9 @@ int launch_mfma(const GemmArgs& a, hipStream_t stream);  // conv_mfma.hip
 
 int launch_tall(const GemmArgs& a, hipStream_t stream);  // conv_tall.hip
 
-int launch_split(const GemmArgs& a, hipStream_t stream);  // conv_split.hip
-
-bool gemm_writes_split(const GemmArgs& a) {
-    if (a.force_valu || a.out_type != SESSD_FLOAT || (reinterpret_cast<uintptr_t>(a.in_feat) | reinterpret_cast<uintptr_t>(a.out_feat)) & 15)
-        return false;
-    if (!a.fp32_mfma && a.w_split && a.in_split && gemm_runs_split(a.K, a.cin, a.cout, a.in_type, a.out_type)) return true;
-    return a.w_packed && gemm_runs_on_mfma(a.K, a.cin, a.cout, a.in_type, a.out_type);
-}
-
 int launch_gather_gemm(const GemmArgs& a, hipStream_t stream) {
     if (!a.force_valu) {  // FP16 3x3x3 layers from 32 channels up: the tall-tile kernel
         const int rc = launch_tall(a, stream);
-        if (rc != SESSD_E_UNSUPPORTED) return rc;
-    }
-    if (!a.force_valu && !a.fp32_mfma) {  // FP32 layers up to 64 channels: three BF16 parts per operand
-        const int rc = launch_split(a, stream);
         if (rc != SESSD_E_UNSUPPORTED) return rc;
     }
     if (!a.force_valu) {

@@ -155,7 +155,7 @@ __global__ void __launch_bounds__(kWaves * 64, min_waves_per_simd(CIN, COUT))
 conv_mfma(const T* __restrict__ in, TO* __restrict__ out, const void* __restrict__ Wp,
           const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
           const float* __restrict__ scale, const float* __restrict__ shift, int relu, int write_pad,
-          int num_cu, const int32_t* __restrict__ tiles, DenseTarget dt, void* __restrict__ out_split) {
+          int num_cu, const int32_t* __restrict__ tiles, DenseTarget dt) {
     using C = Chunk<T, CIN>;
     using Vec = typename C::Vec;
     constexpr int G = CIN / C::kChannels;  // K-chunks of the inner dimension
@@ -447,9 +447,6 @@ conv_mfma(const T* __restrict__ in, TO* __restrict__ out, const void* __restrict
             o[e] = s;
         }
         store4(out + (size_t)(row0 + r) * COUT + ec4, o);
-        if constexpr (sizeof(TO) == 4) {  // FP32 rows also in split form, for a next layer on the split-BF16 kernel
-            if (out_split) store_split4(out_split, row0 + r, COUT, ec4, o);
-        }
         if (dt.dense) {  // the sparse2Dense scatter of this row, fused (uniform branch)
             const int4 cc = reinterpret_cast<const int4*>(dt.coors)[row0 + r];  // (b,z,y,x)
             if (cc.x != 0 || cc.y < 0 || cc.y >= dt.D || cc.z < 0 || cc.z >= dt.H || cc.w < 0 || cc.w >= dt.W) {
@@ -492,7 +489,7 @@ int launch(const GemmArgs& a, hipStream_t stream) {
     hipLaunchKernelGGL((conv_mfma<T, CIN, COUT, TO>), dim3(blocks), dim3(kWaves * 64), 0, stream,
                        static_cast<const T*>(a.in_feat), static_cast<TO*>(a.out_feat), a.w_packed, a.nbr,
                        a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows, num_cu, a.tiles,
-                       a.dense, a.out_type == SESSD_FLOAT ? a.out_split : nullptr);
+                       a.dense);
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;
 }

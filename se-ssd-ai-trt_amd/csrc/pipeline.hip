@@ -44,7 +44,6 @@ struct ConvStage {
     std::unique_ptr<SubmConv3dLayerPlugin> subm;
     std::unique_ptr<SparseConv3dLayerPlugin> sparse;
     DeviceBuffer ws, feat, coors, num;  // coors/num only for sparse layers (they produce new ones)
-    DeviceBuffer split_out;             // `feat` in split form, when the next layer runs on the split-BF16 kernel
     int rulebook_from = -1;             // SubM layer whose workspace holds this layer's rulebook
     sessd_tensor_desc in_desc[3], out_desc[3];
     void* coors_ptr = nullptr;  // coordinates valid AFTER this layer
@@ -112,31 +111,6 @@ struct Pipeline {
         if (ev_fill) (void)hipEventDestroy(ev_fill);
         if (aux) (void)hipStreamDestroy(aux);
         if (aux_fill) (void)hipStreamDestroy(aux_fill);
-    }
-
-    // The gather-GEMM of layer l on `stream`: input rows `feat` (the previous layer's, whose split form is passed
-    // along when that layer keeps one), output rows into the stage's tensors -- in split form as well when the
-    // next layer wants them, by the GEMM's own epilogue where its kernel can, by a conversion launch otherwise.
-    int enqueueLayerGemm(size_t l, const void* feat, const int32_t* num_in, hipStream_t stream, const DenseTarget* dt) {
-        ConvStage& st = *stages[l];
-        const void* in_split = l > 0 ? stages[l - 1]->split_out.p : nullptr;
-        void* out_split = st.split_out.p;
-        const int owner = st.rulebook_from >= 0 ? st.rulebook_from : (int)l;
-        const int32_t* num_out = st.subm ? num_in : static_cast<const int32_t*>(st.num.p);
-        bool writes;
-        if (st.subm) {
-            writes = st.subm->gemmWritesSplit(feat, st.feat.p, in_split);
-            SESSD_TRY(st.subm->enqueueGemm(feat, st.feat.p, num_in, stages[owner]->ws.p, stream, dt, in_split,
-                                           writes ? out_split : nullptr));
-        } else {
-            writes = st.sparse->gemmWritesSplit(feat, st.feat.p, in_split);
-            SESSD_TRY(st.sparse->enqueueGemm(feat, st.feat.p, num_out, st.ws.p, stream, dt, in_split,
-                                             writes ? out_split : nullptr));
-        }
-        if (out_split && !writes)
-            SESSD_TRY(launch_split_rows(static_cast<const float*>(st.feat.p), out_split, num_out, max_voxels,
-                                        st.spec.out_channel, stream));
-        return SESSD_OK;
     }
 
     // The rulebooks depend only on coordinates, the GEMMs on rulebooks + features.  The coordinate chain
@@ -255,8 +229,11 @@ struct Pipeline {
                 dt = s2d->denseTarget(dense, oc, s2d_ws.p);
                 scattered = true;
             }
-            SESSD_TRY(enqueueLayerGemm(l, feat, num, stream, fuse ? &dt : nullptr));
-            if (st.sparse) {
+            if (st.subm) {
+                SESSD_TRY(st.subm->enqueueGemm(feat, st.feat.p, num, stages[owner]->ws.p, stream, fuse ? &dt : nullptr));
+            } else {
+                SESSD_TRY(st.sparse->enqueueGemm(feat, st.feat.p, static_cast<const int32_t*>(st.num.p), st.ws.p, stream,
+                                                 fuse ? &dt : nullptr));
                 coors = static_cast<const int32_t*>(st.coors.p);
                 num = static_cast<const int32_t*>(st.num.p);
             }
@@ -282,19 +259,18 @@ struct Pipeline {
         const void* feat = vg_voxels.p;
         const void* coors = vg_coors.p;
         const void* num = vg_num.p;
-        for (size_t l = 0; l < stages.size(); ++l) {  // every layer: its rulebook (unless shared), then its GEMM
-            ConvStage* st = stages[l].get();
+        for (auto& st : stages) {
+            const void* in[3] = {feat, coors, num};
             if (st->subm) {
-                if (st->rulebook_from < 0)
-                    SESSD_TRY(st->subm->enqueueBuild(static_cast<const int32_t*>(coors), static_cast<const int32_t*>(num),
-                                                     st->ws.p, stream));
+                void* out[1] = {st->feat.p};
+                if (st->rulebook_from >= 0)
+                    SESSD_TRY(st->subm->enqueueShared(st->in_desc, st->out_desc, in, out,
+                                                      stages[st->rulebook_from]->ws.p, stream));
+                else
+                    SESSD_TRY(st->subm->enqueue(st->in_desc, st->out_desc, in, out, st->ws.p, stream));
             } else {
-                SESSD_TRY(st->sparse->enqueueBuild(static_cast<const int32_t*>(coors), static_cast<const int32_t*>(num),
-                                                   static_cast<int32_t*>(st->coors.p), static_cast<int32_t*>(st->num.p),
-                                                   st->ws.p, stream));
-            }
-            SESSD_TRY(enqueueLayerGemm(l, feat, static_cast<const int32_t*>(num), stream, nullptr));
-            if (st->sparse) {
+                void* out[3] = {st->feat.p, st->coors.p, st->num.p};
+                SESSD_TRY(st->sparse->enqueue(st->in_desc, st->out_desc, in, out, st->ws.p, stream));
                 coors = st->coors.p;
                 num = st->num.p;
             }
@@ -415,16 +391,6 @@ static int build_pipeline(const sessd_pipeline_desc& d, Pipeline* P) {
         in_type = ft;
         in_ch = s.out_channel;
         P->stages.push_back(std::move(st));
-    }
-
-    // a layer on the split-BF16 kernel reads its input rows in split form: the layer before it keeps them
-    for (size_t l = 1; l < P->stages.size(); ++l) {
-        ConvStage& st = *P->stages[l];
-        const ConvPluginBase* cp = st.subm ? static_cast<const ConvPluginBase*>(st.subm.get()) : st.sparse.get();
-        if (!cp->gemmOnSplitKernel()) continue;
-        ConvStage& prev = *P->stages[l - 1];
-        SESSD_TRY(prev.split_out.alloc(split_feature_bytes(V, prev.spec.out_channel)));
-        total += prev.split_out.bytes;
     }
 
     if (d.dense.feature_map_channel != in_ch)

@@ -6,7 +6,6 @@
 #include <vector>
 
 #include "common.h"
-#include "kernels.h"
 
 namespace sessd {
 
@@ -68,7 +67,6 @@ class VoxelGeneratorPlugin {
 // Shared by both conv plugins: device weights (+ epilogue), dtype bookkeeping, GEMM dispatch
 // ---------------------------------------------------------------------------------------------
 bool gemm_runs_tall(int K, int cin, int cout, int in_type, int out_type);  // kernels.h
-bool gemm_runs_split(int K, int cin, int cout, int in_type, int out_type);
 // Cin * Cout (of the layer that builds it) from which a rulebook gets equal-work tile cuts.  At 32 x 32 the GEMM
 // measured the same with and without them, and the two launches lengthen the coordinate branch: frame 0.387 -> 0.377 ms.
 constexpr int kTileCutMinWork = 32 * 64;
@@ -94,7 +92,6 @@ class ConvPluginBase {
     float* weights_dev_ = nullptr;     // FP32 [K][Cin][Cout]
     __half* weights_half_dev_ = nullptr;  // FP16 copy of the same layout
     void* weights_packed_dev_ = nullptr;  // MFMA B-operand order (see conv_gemm.hip)
-    void* weights_split_dev_ = nullptr;   // three BF16 parts in MFMA operand order (conv_split.hip), FP32 layers only
     int packed_dtype_ = -1;
     Epilogue epi_;
     int in_type_ = SESSD_FLOAT, out_type_ = SESSD_FLOAT;
@@ -105,28 +102,15 @@ class ConvPluginBase {
   protected:
     // gather-GEMM over the neighbour table nbr[K][max_voxels] (device), rows < *num_out
     // `dense`: also scatter the output rows into the dense tensor of a sparse2Dense step (MFMA kernel only)
-    // `in_split` / `out_split`: the input rows in split form (needed by the split-BF16 kernel; without them an FP32
-    // layer runs on the FP32 MFMA kernel) / where to write the output rows in that form as well (kernels.h)
     int runGemm(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* tiles,
-                const int32_t* num_out, hipStream_t stream, const DenseTarget* dense = nullptr,
-                const void* in_split = nullptr, void* out_split = nullptr);
-    GemmArgs gemmArgs(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* tiles,
-                      const int32_t* num_out, const DenseTarget* dense, const void* in_split, void* out_split) const;
+                const int32_t* num_out, hipStream_t stream, const DenseTarget* dense = nullptr);
     // whether a rulebook built by this layer gets equal-work tile cuts: worth two small launches when the
     // GEMM runs on the matrix cores and is not tiny
     bool wantTileCuts() const {
         return weights_packed_dev_ != nullptr && !(flags_ & SESSD_FLAG_FORCE_VALU) &&
                in_channel_ * out_channel_ >= kTileCutMinWork &&
-               !gemm_runs_tall(kernel_volume_, in_channel_, out_channel_, in_type_, out_type_) && !gemmOnSplitKernel();
+               !gemm_runs_tall(kernel_volume_, in_channel_, out_channel_, in_type_, out_type_);
     }
-  public:
-    // whether this layer, given its input rows in split form, runs on the split-BF16 kernel (conv_split.hip)
-    bool gemmOnSplitKernel() const {
-        return weights_split_dev_ != nullptr && !(flags_ & (SESSD_FLAG_FORCE_VALU | SESSD_FLAG_FP32_MFMA)) &&
-               gemm_runs_split(kernel_volume_, in_channel_, out_channel_, in_type_, out_type_);
-    }
-
-  protected:
     // tile height those cuts aim at: the capacity of this layer's own GEMM kernel
     int tileRows() const;
     int exportRulebook(const int32_t* nbr, const int32_t* num_out, void* scratch,
@@ -165,10 +149,7 @@ class SubmConv3dLayerPlugin : public ConvPluginBase {
     MirrorInit mirrorInit(void* workspace) const;
     void collectFill(void* workspace, FillArgs& f, bool own_table = true) const;
     int enqueueGemm(const void* in_feat, void* out_feat, const int32_t* voxel_num,
-                    const void* rulebook_workspace, hipStream_t stream, const DenseTarget* dense = nullptr,
-                    const void* in_split = nullptr, void* out_split = nullptr);
-    // whether the GEMM, launched with these split pointers, writes out_split itself (else: launch_split_rows)
-    bool gemmWritesSplit(const void* in_feat, void* out_feat, const void* in_split) const;
+                    const void* rulebook_workspace, hipStream_t stream, const DenseTarget* dense = nullptr);
     int exportRulebook(const void* workspace, int32_t* indice_pairs, uint32_t* indice_num,
                        hipStream_t stream) const;
     int countPairs(const void* workspace, uint32_t* indice_num, hipStream_t stream) const;
@@ -209,9 +190,7 @@ class SparseConv3dLayerPlugin : public ConvPluginBase {
     HashTable cellTable(void* workspace) const;
     void collectFill(void* workspace, int32_t* out_coors, FillArgs& f) const;
     int enqueueGemm(const void* in_feat, void* out_feat, const int32_t* out_num, const void* workspace,
-                    hipStream_t stream, const DenseTarget* dense = nullptr, const void* in_split = nullptr,
-                    void* out_split = nullptr);
-    bool gemmWritesSplit(const void* in_feat, void* out_feat, const void* in_split) const;
+                    hipStream_t stream, const DenseTarget* dense = nullptr);
     size_t getSerializationSize() const;
     void serialize(void* buffer) const;
     size_t statusOffset() const;

@@ -185,7 +185,6 @@ struct SparseConv3dLayerPlugin::Layout {
     void* export_scratch;
     int32_t* tiles;  // equal-work tile cuts of the rulebook (tile_cut.hip); first word 0 = none
     int32_t* meta;
-    void* split_in;  // the input rows in split form (layers that run on the split-BF16 kernel), or null
     uint32_t cap;
     int Kc;
     int n_blocks;
@@ -227,9 +226,6 @@ SparseConv3dLayerPlugin::Layout SparseConv3dLayerPlugin::carve(void* workspace) 
     L.tiles = reinterpret_cast<int32_t*>(c.take<uint8_t>(tile_cut_bytes(max_voxels_)));
     L.meta_offset = c.offset;
     L.meta = c.take<int32_t>(4);
-    L.split_in = nullptr;
-    if (gemm_runs_split(kernel_volume_, in_channel_, out_channel_, in_type_, out_type_))
-        L.split_in = c.take<uint8_t>(split_feature_bytes(max_voxels_, in_channel_));
     L.total = c.total();
     return L;
 }
@@ -414,15 +410,10 @@ HashTable SparseConv3dLayerPlugin::cellTable(void* workspace) const {
 }
 
 int SparseConv3dLayerPlugin::enqueueGemm(const void* in_feat, void* out_feat, const int32_t* out_num,
-                                         const void* workspace, hipStream_t stream, const DenseTarget* dense,
-                                         const void* in_split, void* out_split) {
+                                         const void* workspace, hipStream_t stream, const DenseTarget* dense) {
     if (!in_feat || !out_feat || !out_num || !workspace) return fail(SESSD_E_INVALID, "sparseconv3d.gemm: null pointer");
     const Layout L = carve(const_cast<void*>(workspace));
-    return runGemm(in_feat, out_feat, L.nbr, L.tiles, out_num, stream, dense, in_split, out_split);
-}
-
-bool SparseConv3dLayerPlugin::gemmWritesSplit(const void* in_feat, void* out_feat, const void* in_split) const {
-    return gemm_writes_split(gemmArgs(in_feat, out_feat, nullptr, nullptr, nullptr, nullptr, in_split, nullptr));
+    return runGemm(in_feat, out_feat, L.nbr, L.tiles, out_num, stream, dense);
 }
 
 int SparseConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
@@ -434,13 +425,7 @@ int SparseConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const s
     int32_t* out_num = static_cast<int32_t*>(outputs[2]);
     SESSD_TRY(enqueueBuild(static_cast<const int32_t*>(inputs[1]), static_cast<const int32_t*>(inputs[2]),
                            static_cast<int32_t*>(outputs[1]), out_num, workspace, stream));
-    const void* in_split = nullptr;
-    if (gemmOnSplitKernel()) {  // the caller's rows are plain FP32: their split form goes into the workspace
-        in_split = carve(workspace).split_in;
-        SESSD_TRY(launch_split_rows(static_cast<const float*>(inputs[0]), const_cast<void*>(in_split),
-                                    static_cast<const int32_t*>(inputs[2]), max_voxels_, in_channel_, stream));
-    }
-    return enqueueGemm(inputs[0], outputs[0], out_num, workspace, stream, nullptr, in_split);
+    return enqueueGemm(inputs[0], outputs[0], out_num, workspace, stream);
 }
 
 int SparseConv3dLayerPlugin::exportRulebook(const void* workspace, int32_t* indice_pairs, uint32_t* indice_num,

@@ -112,7 +112,6 @@ struct SubmConv3dLayerPlugin::Layout {
     void* export_scratch;
     int32_t* tiles;  // equal-work tile cuts of the rulebook (tile_cut.hip); first word 0 = none
     int32_t* meta;  // [0] status word, [1] active rows of the last enqueue
-    void* split_in;  // the input rows in split form (layers that run on the split-BF16 kernel), or null
     uint32_t cap;
     size_t meta_offset;
     size_t total;
@@ -129,9 +128,6 @@ SubmConv3dLayerPlugin::Layout SubmConv3dLayerPlugin::carve(void* workspace) cons
     L.tiles = reinterpret_cast<int32_t*>(c.take<uint8_t>(tile_cut_bytes(max_voxels_)));
     L.meta_offset = c.offset;
     L.meta = c.take<int32_t>(4);
-    L.split_in = nullptr;
-    if (gemm_runs_split(kernel_volume_, in_channel_, out_channel_, in_type_, out_type_))
-        L.split_in = c.take<uint8_t>(split_feature_bytes(max_voxels_, in_channel_));
     L.total = c.total();
     return L;
 }
@@ -305,15 +301,11 @@ MirrorInit SubmConv3dLayerPlugin::mirrorInit(void* workspace) const {
 
 int SubmConv3dLayerPlugin::enqueueGemm(const void* in_feat, void* out_feat, const int32_t* voxel_num,
                                        const void* rulebook_workspace, hipStream_t stream,
-                                       const DenseTarget* dense, const void* in_split, void* out_split) {
+                                       const DenseTarget* dense) {
     if (!in_feat || !out_feat || !voxel_num || !rulebook_workspace)
         return fail(SESSD_E_INVALID, "submconv3d.gemm: null pointer");
     const Layout L = carve(const_cast<void*>(rulebook_workspace));
-    return runGemm(in_feat, out_feat, L.nbr, L.tiles, voxel_num, stream, dense, in_split, out_split);
-}
-
-bool SubmConv3dLayerPlugin::gemmWritesSplit(const void* in_feat, void* out_feat, const void* in_split) const {
-    return gemm_writes_split(gemmArgs(in_feat, out_feat, nullptr, nullptr, nullptr, nullptr, in_split, nullptr));
+    return runGemm(in_feat, out_feat, L.nbr, L.tiles, voxel_num, stream, dense);
 }
 
 int SubmConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
@@ -324,13 +316,7 @@ int SubmConv3dLayerPlugin::enqueue(const sessd_tensor_desc* inputDesc, const ses
     if (!workspace) return fail(SESSD_E_INVALID, "submconv3d.enqueue: workspace is null");
     const int32_t* voxel_num = static_cast<const int32_t*>(inputs[2]);
     SESSD_TRY(enqueueBuild(static_cast<const int32_t*>(inputs[1]), voxel_num, workspace, stream));
-    const void* in_split = nullptr;
-    if (gemmOnSplitKernel()) {  // the caller's rows are plain FP32: their split form goes into the workspace
-        in_split = carve(workspace).split_in;
-        SESSD_TRY(launch_split_rows(static_cast<const float*>(inputs[0]), const_cast<void*>(in_split), voxel_num,
-                                    max_voxels_, in_channel_, stream));
-    }
-    return enqueueGemm(inputs[0], outputs[0], voxel_num, workspace, stream, nullptr, in_split);
+    return enqueueGemm(inputs[0], outputs[0], voxel_num, workspace, stream);
 }
 
 int SubmConv3dLayerPlugin::enqueueShared(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,

@@ -503,10 +503,9 @@ class Pipeline:
                  feature_dtype="fp32", relu=True, share_rulebooks=True, skip_pad_rows=False, use_graph=False,
                  dense_size_xyz=B.DENSE_SIZE_XYZ, max_pts_per_voxel=B.MAX_NUM_POINTS_PER_VOXEL,
                  use_epilogue=True, overlap_streams=False, voxel_cap=None, dense_padding=(0, 0, 0, 0),
-                 force_valu=False, frames_in_flight=0, fp32_mfma=False):
+                 force_valu=False, frames_in_flight=0):
         """max_voxels = rows of every conv-layer tensor; voxel_cap (default: max_voxels) = the voxelizer's
-        own limit.  force_valu: every gather-GEMM on the shape-agnostic VALU kernel (cross-checks).
-        fp32_mfma: FP32 layers on the FP32 matrix instructions instead of the split-BF16 kernel."""
+        own limit.  force_valu: every gather-GEMM on the shape-agnostic VALU kernel (cross-checks)."""
         torch = _torch()
         self.layers = list(layers)
         self.max_points, self.max_voxels = max_points, max_voxels
@@ -538,8 +537,7 @@ class Pipeline:
         c_last = self.layers[-1].cout if n else 4
         d.dense = B.dense_desc(dense_size_xyz, c_last)
         d.share_rulebooks = int(share_rulebooks)
-        d.flags = (D.SESSD_FLAG_SKIP_PAD_ROWS if skip_pad_rows else 0) | (D.SESSD_FLAG_FORCE_VALU if force_valu else 0) | \
-                  (D.SESSD_FLAG_FP32_MFMA if fp32_mfma else 0)
+        d.flags = (D.SESSD_FLAG_SKIP_PAD_ROWS if skip_pad_rows else 0) | (D.SESSD_FLAG_FORCE_VALU if force_valu else 0)
         d.use_graph = int(use_graph)
         d.overlap_streams = int(overlap_streams)
         d.frames_in_flight = int(frames_in_flight)

@@ -17,7 +17,6 @@ SESSD_STATUS_BAD_COORD = 4
 
 SESSD_FLAG_SKIP_PAD_ROWS = 1
 SESSD_FLAG_FORCE_VALU = 2
-SESSD_FLAG_FP32_MFMA = 4
 
 SESSD_LAYER_SUBM = 0
 SESSD_LAYER_SPARSE = 1
