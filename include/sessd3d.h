@@ -457,6 +457,10 @@ int sessd_pipeline_enqueue(sessd_pipeline* h, const void* points, const void* po
  * last.  With frames_in_flight < 2: submit = enqueue, join does nothing. */
 int sessd_pipeline_submit(sessd_pipeline* h, const void* points, const void* points_size, void* dense,
                           sessd_stream_t stream, int64_t* ticket);
+/* (join with stream = SESSD_STREAM_NONE blocks the calling thread, as sessd_pipeline_wait does.  With frames in
+ * flight, sessd_pipeline_status / _layer_stats first make `stream` wait for the last submitted frame; a caller
+ * that reads tensors of sessd_pipeline_layer_io itself has to join that frame first; sessd_pipeline_enqueue_timed
+ * is refused.) */
 int sessd_pipeline_join(sessd_pipeline* h, int64_t ticket, sessd_stream_t stream);
 /* join for a host loop: blocks the calling thread (not a stream) until the frame of `ticket` is complete.  A
  * stream-side join puts a wait into the caller's stream, and where that stream shares a hardware queue with

@@ -36,17 +36,21 @@ int sessd_copy_to_host(void* dst_host, const void* src_device, size_t bytes, ses
 // ------------------------------------------------------------------ voxelgen
 int sessd_voxelgen_create(const sessd_voxelgen_desc* desc, sessd_voxelgen** out) {
     NEED(desc && out, "null argument");
-    VoxelGeneratorPlugin* p = nullptr;
-    SESSD_TRY(VoxelGeneratorPlugin::create(*desc, &p));
-    *out = reinterpret_cast<sessd_voxelgen*>(p);
-    return SESSD_OK;
+    return guarded(__func__, [&]() -> int {
+        VoxelGeneratorPlugin* p = nullptr;
+        SESSD_TRY(VoxelGeneratorPlugin::create(*desc, &p));
+        *out = reinterpret_cast<sessd_voxelgen*>(p);
+        return SESSD_OK;
+    });
 }
 int sessd_voxelgen_deserialize(const void* bytes, size_t n, sessd_voxelgen** out) {
     NEED(out, "null argument");
-    VoxelGeneratorPlugin* p = nullptr;
-    SESSD_TRY(VoxelGeneratorPlugin::deserialize(bytes, n, &p));
-    *out = reinterpret_cast<sessd_voxelgen*>(p);
-    return SESSD_OK;
+    return guarded(__func__, [&]() -> int {
+        VoxelGeneratorPlugin* p = nullptr;
+        SESSD_TRY(VoxelGeneratorPlugin::deserialize(bytes, n, &p));
+        *out = reinterpret_cast<sessd_voxelgen*>(p);
+        return SESSD_OK;
+    });
 }
 size_t sessd_voxelgen_serialization_size(const sessd_voxelgen* h) { return h ? CH_VG(h)->getSerializationSize() : 0; }
 int sessd_voxelgen_serialize(const sessd_voxelgen* h, void* buf) {
@@ -101,17 +105,21 @@ void sessd_voxelgen_destroy(sessd_voxelgen* h) { delete H_VG(h); }
 // ------------------------------------------------------------------ submconv3d
 int sessd_submconv3d_create(const sessd_submconv3d_desc* desc, const float* weights, sessd_submconv3d** out) {
     NEED(desc && weights && out, "null argument");
-    SubmConv3dLayerPlugin* p = nullptr;
-    SESSD_TRY(SubmConv3dLayerPlugin::create(*desc, weights, &p));
-    *out = reinterpret_cast<sessd_submconv3d*>(p);
-    return SESSD_OK;
+    return guarded(__func__, [&]() -> int {
+        SubmConv3dLayerPlugin* p = nullptr;
+        SESSD_TRY(SubmConv3dLayerPlugin::create(*desc, weights, &p));
+        *out = reinterpret_cast<sessd_submconv3d*>(p);
+        return SESSD_OK;
+    });
 }
 int sessd_submconv3d_deserialize(const void* bytes, size_t n, sessd_submconv3d** out) {
     NEED(out, "null argument");
-    SubmConv3dLayerPlugin* p = nullptr;
-    SESSD_TRY(SubmConv3dLayerPlugin::deserialize(bytes, n, &p));
-    *out = reinterpret_cast<sessd_submconv3d*>(p);
-    return SESSD_OK;
+    return guarded(__func__, [&]() -> int {
+        SubmConv3dLayerPlugin* p = nullptr;
+        SESSD_TRY(SubmConv3dLayerPlugin::deserialize(bytes, n, &p));
+        *out = reinterpret_cast<sessd_submconv3d*>(p);
+        return SESSD_OK;
+    });
 }
 size_t sessd_submconv3d_serialization_size(const sessd_submconv3d* h) {
     return h ? CH_SUBM(h)->getSerializationSize() : 0;
@@ -124,7 +132,7 @@ int sessd_submconv3d_serialize(const sessd_submconv3d* h, void* buf) {
 int sessd_submconv3d_configure(sessd_submconv3d* h, const sessd_tensor_desc* in, int nIn,
                                const sessd_tensor_desc* out, int nOut) {
     NEED(h, "null handle");
-    return H_SUBM(h)->configurePlugin(in, nIn, out, nOut);
+    return guarded(__func__, [&]() -> int { return H_SUBM(h)->configurePlugin(in, nIn, out, nOut); });
 }
 size_t sessd_submconv3d_workspace_size(const sessd_submconv3d* h, const sessd_tensor_desc* in, int nIn,
                                        const sessd_tensor_desc* out, int nOut) {
@@ -150,7 +158,9 @@ int sessd_submconv3d_export_rulebook(const sessd_submconv3d* h, const void* work
 }
 int sessd_submconv3d_set_epilogue(sessd_submconv3d* h, const float* scale, const float* shift, int relu) {
     NEED(h, "null handle");
-    return H_SUBM(h)->setEpilogue(scale, shift, relu);
+    return guarded(__func__, [&]() -> int {
+        return H_SUBM(h)->setEpilogue(scale, shift, relu);
+    });
 }
 int sessd_submconv3d_set_flags(sessd_submconv3d* h, int32_t flags) {
     NEED(h, "null handle");
@@ -167,17 +177,21 @@ void sessd_submconv3d_destroy(sessd_submconv3d* h) { delete H_SUBM(h); }
 // ------------------------------------------------------------------ sparseconv3d
 int sessd_sparseconv3d_create(const sessd_sparseconv3d_desc* desc, const float* weights, sessd_sparseconv3d** out) {
     NEED(desc && weights && out, "null argument");
-    SparseConv3dLayerPlugin* p = nullptr;
-    SESSD_TRY(SparseConv3dLayerPlugin::create(*desc, weights, &p));
-    *out = reinterpret_cast<sessd_sparseconv3d*>(p);
-    return SESSD_OK;
+    return guarded(__func__, [&]() -> int {
+        SparseConv3dLayerPlugin* p = nullptr;
+        SESSD_TRY(SparseConv3dLayerPlugin::create(*desc, weights, &p));
+        *out = reinterpret_cast<sessd_sparseconv3d*>(p);
+        return SESSD_OK;
+    });
 }
 int sessd_sparseconv3d_deserialize(const void* bytes, size_t n, sessd_sparseconv3d** out) {
     NEED(out, "null argument");
-    SparseConv3dLayerPlugin* p = nullptr;
-    SESSD_TRY(SparseConv3dLayerPlugin::deserialize(bytes, n, &p));
-    *out = reinterpret_cast<sessd_sparseconv3d*>(p);
-    return SESSD_OK;
+    return guarded(__func__, [&]() -> int {
+        SparseConv3dLayerPlugin* p = nullptr;
+        SESSD_TRY(SparseConv3dLayerPlugin::deserialize(bytes, n, &p));
+        *out = reinterpret_cast<sessd_sparseconv3d*>(p);
+        return SESSD_OK;
+    });
 }
 size_t sessd_sparseconv3d_serialization_size(const sessd_sparseconv3d* h) {
     return h ? CH_SP(h)->getSerializationSize() : 0;
@@ -190,7 +204,7 @@ int sessd_sparseconv3d_serialize(const sessd_sparseconv3d* h, void* buf) {
 int sessd_sparseconv3d_configure(sessd_sparseconv3d* h, const sessd_tensor_desc* in, int nIn,
                                  const sessd_tensor_desc* out, int nOut) {
     NEED(h, "null handle");
-    return H_SP(h)->configurePlugin(in, nIn, out, nOut);
+    return guarded(__func__, [&]() -> int { return H_SP(h)->configurePlugin(in, nIn, out, nOut); });
 }
 size_t sessd_sparseconv3d_workspace_size(const sessd_sparseconv3d* h, const sessd_tensor_desc* in, int nIn,
                                          const sessd_tensor_desc* out, int nOut) {
@@ -209,7 +223,9 @@ int sessd_sparseconv3d_export_rulebook(const sessd_sparseconv3d* h, const void* 
 }
 int sessd_sparseconv3d_set_epilogue(sessd_sparseconv3d* h, const float* scale, const float* shift, int relu) {
     NEED(h, "null handle");
-    return H_SP(h)->setEpilogue(scale, shift, relu);
+    return guarded(__func__, [&]() -> int {
+        return H_SP(h)->setEpilogue(scale, shift, relu);
+    });
 }
 int sessd_sparseconv3d_set_flags(sessd_sparseconv3d* h, int32_t flags) {
     NEED(h, "null handle");
@@ -226,17 +242,21 @@ void sessd_sparseconv3d_destroy(sessd_sparseconv3d* h) { delete H_SP(h); }
 // ------------------------------------------------------------------ sparse2dense
 int sessd_sparse2dense_create(const sessd_sparse2dense_desc* desc, sessd_sparse2dense** out) {
     NEED(desc && out, "null argument");
-    Sparse2DensePlugin* p = nullptr;
-    SESSD_TRY(Sparse2DensePlugin::create(*desc, &p));
-    *out = reinterpret_cast<sessd_sparse2dense*>(p);
-    return SESSD_OK;
+    return guarded(__func__, [&]() -> int {
+        Sparse2DensePlugin* p = nullptr;
+        SESSD_TRY(Sparse2DensePlugin::create(*desc, &p));
+        *out = reinterpret_cast<sessd_sparse2dense*>(p);
+        return SESSD_OK;
+    });
 }
 int sessd_sparse2dense_deserialize(const void* bytes, size_t n, sessd_sparse2dense** out) {
     NEED(out, "null argument");
-    Sparse2DensePlugin* p = nullptr;
-    SESSD_TRY(Sparse2DensePlugin::deserialize(bytes, n, &p));
-    *out = reinterpret_cast<sessd_sparse2dense*>(p);
-    return SESSD_OK;
+    return guarded(__func__, [&]() -> int {
+        Sparse2DensePlugin* p = nullptr;
+        SESSD_TRY(Sparse2DensePlugin::deserialize(bytes, n, &p));
+        *out = reinterpret_cast<sessd_sparse2dense*>(p);
+        return SESSD_OK;
+    });
 }
 size_t sessd_sparse2dense_serialization_size(const sessd_sparse2dense* h) {
     return h ? CH_S2D(h)->getSerializationSize() : 0;

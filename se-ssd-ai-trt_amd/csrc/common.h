@@ -8,6 +8,8 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <new>
+#include <stdexcept>
 #include <string>
 
 #include "../../include/sessd3d.h"
@@ -28,6 +30,23 @@ int fail(int code, const char* fmt, ...);
             return ::sessd::fail(SESSD_E_HIP, "%s:%d: %s -> %s", __FILE__, __LINE__, #expr,      \
                                  hipGetErrorString(e__));                                        \
     } while (0)
+
+// The body of an extern "C" entry point that can allocate on the host (new, std::vector, std::string): no C++
+// exception may cross the C boundary, so what the body throws becomes an error code and a message.
+template <typename F>
+inline int guarded(const char* who, F&& body) noexcept {
+    try {
+        return body();
+    } catch (const std::bad_alloc&) {
+        return fail(SESSD_E_NOMEM, "%s: out of host memory", who);
+    } catch (const std::length_error&) {
+        return fail(SESSD_E_NOMEM, "%s: a size beyond what host memory can hold", who);
+    } catch (const std::exception& e) {
+        return fail(SESSD_E_INVALID, "%s: %s", who, e.what());
+    } catch (...) {
+        return fail(SESSD_E_INVALID, "%s: unknown C++ exception", who);
+    }
+}
 
 #define SESSD_TRY(expr)                  \
     do {                                 \

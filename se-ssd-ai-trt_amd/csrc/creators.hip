@@ -85,6 +85,9 @@ int find_field(const sessd_plugin_field_collection* fc, const Registry& r, const
         if (spec && f.type != spec->type)
             return fail(SESSD_E_INVALID, "%s: field '%s' has type %d, the creator reads type %d", r.plugin_name, name, f.type,
                         spec->type);
+        if (spec && spec->length > 1 && f.length != 1 && f.length < spec->length)
+            return fail(SESSD_E_INVALID, "%s: field '%s' declares %d elements, the creator reads %d", r.plugin_name, name,
+                        f.length, spec->length);
         *data = f.data;
         if (length) *length = f.length;
         return SESSD_OK;
@@ -152,7 +155,7 @@ const sessd_plugin_field_collection* sessd_plugin_field_names(const char* plugin
     return &r->fc;
 }
 
-int sessd_plugin_create(const char* plugin_name, const sessd_plugin_field_collection* fc, void** handle) {
+static int plugin_create_unguarded(const char* plugin_name, const sessd_plugin_field_collection* fc, void** handle) {
     if (!plugin_name || !fc || !handle || (fc->nbFields > 0 && !fc->fields) || fc->nbFields < 0)
         return fail(SESSD_E_INVALID, "plugin_create: null argument");
     const Registry* rp = registry(plugin_name);
@@ -217,44 +220,56 @@ int sessd_plugin_create(const char* plugin_name, const sessd_plugin_field_collec
     return sessd_sparseconv3d_create(&d, w, reinterpret_cast<sessd_sparseconv3d**>(handle));
 }
 
+int sessd_plugin_create(const char* plugin_name, const sessd_plugin_field_collection* fc, void** handle) {
+    return guarded(__func__, [&]() -> int { return plugin_create_unguarded(plugin_name, fc, handle); });
+}
+
 // clone(): the reference builds a new plugin from the members of the old one, device weights included
 // (submConv3dlayer.cu:188-196); here the copy also carries what this library adds to a plugin (epilogue, flags,
 // the configured tensor types, the dense border).  The serialised form is the member list, so a clone is a
 // deserialisation of it plus the members that are not serialised.
 int sessd_voxelgen_clone(const sessd_voxelgen* h, sessd_voxelgen** out) {
     if (!h || !out) return fail(SESSD_E_INVALID, "voxelgen_clone: null argument");
-    const auto* src = reinterpret_cast<const VoxelGeneratorPlugin*>(h);
-    std::vector<char> blob(src->getSerializationSize());
-    src->serialize(blob.data());
-    VoxelGeneratorPlugin* p = nullptr;
-    SESSD_TRY(VoxelGeneratorPlugin::deserialize(blob.data(), blob.size(), &p));
-    p->flags_ = src->flags_;
-    p->lastMaxPoints_ = src->lastMaxPoints_;
-    *out = reinterpret_cast<sessd_voxelgen*>(p);
-    return SESSD_OK;
+    return guarded(__func__, [&]() -> int {
+        const auto* src = reinterpret_cast<const VoxelGeneratorPlugin*>(h);
+        std::vector<char> blob(src->getSerializationSize());
+        src->serialize(blob.data());
+        VoxelGeneratorPlugin* p = nullptr;
+        SESSD_TRY(VoxelGeneratorPlugin::deserialize(blob.data(), blob.size(), &p));
+        p->flags_ = src->flags_;
+        p->lastMaxPoints_ = src->lastMaxPoints_;
+        *out = reinterpret_cast<sessd_voxelgen*>(p);
+        return SESSD_OK;
+    });
 }
 
 int sessd_submconv3d_clone(const sessd_submconv3d* h, sessd_submconv3d** out) {
     if (!h || !out) return fail(SESSD_E_INVALID, "submconv3d_clone: null argument");
-    return clone_conv(reinterpret_cast<const SubmConv3dLayerPlugin*>(h), reinterpret_cast<SubmConv3dLayerPlugin**>(out));
+    return guarded(__func__, [&]() -> int {
+        return clone_conv(reinterpret_cast<const SubmConv3dLayerPlugin*>(h), reinterpret_cast<SubmConv3dLayerPlugin**>(out));
+    });
 }
 
 int sessd_sparseconv3d_clone(const sessd_sparseconv3d* h, sessd_sparseconv3d** out) {
     if (!h || !out) return fail(SESSD_E_INVALID, "sparseconv3d_clone: null argument");
-    return clone_conv(reinterpret_cast<const SparseConv3dLayerPlugin*>(h), reinterpret_cast<SparseConv3dLayerPlugin**>(out));
+    return guarded(__func__, [&]() -> int {
+        return clone_conv(reinterpret_cast<const SparseConv3dLayerPlugin*>(h), reinterpret_cast<SparseConv3dLayerPlugin**>(out));
+    });
 }
 
 int sessd_sparse2dense_clone(const sessd_sparse2dense* h, sessd_sparse2dense** out) {
     if (!h || !out) return fail(SESSD_E_INVALID, "sparse2dense_clone: null argument");
-    const auto* src = reinterpret_cast<const Sparse2DensePlugin*>(h);
-    std::vector<char> blob(src->getSerializationSize());
-    src->serialize(blob.data());
-    Sparse2DensePlugin* p = nullptr;
-    SESSD_TRY(Sparse2DensePlugin::deserialize(blob.data(), blob.size(), &p));
-    p->in_type_ = src->in_type_;
-    p->out_type_ = src->out_type_;
-    *out = reinterpret_cast<sessd_sparse2dense*>(p);
-    return SESSD_OK;
+    return guarded(__func__, [&]() -> int {
+        const auto* src = reinterpret_cast<const Sparse2DensePlugin*>(h);
+        std::vector<char> blob(src->getSerializationSize());
+        src->serialize(blob.data());
+        Sparse2DensePlugin* p = nullptr;
+        SESSD_TRY(Sparse2DensePlugin::deserialize(blob.data(), blob.size(), &p));
+        p->in_type_ = src->in_type_;
+        p->out_type_ = src->out_type_;
+        *out = reinterpret_cast<sessd_sparse2dense*>(p);
+        return SESSD_OK;
+    });
 }
 
 }  // extern "C"

@@ -471,8 +471,7 @@ int sessd_reference_backbone(sessd_layer_spec* layers, int max_layers, sessd_vox
     return n;
 }
 
-int sessd_pipeline_create(const sessd_pipeline_desc* desc, sessd_pipeline** out) {
-    if (!desc || !out) return fail(SESSD_E_INVALID, "pipeline_create: null argument");
+static int pipeline_create_unguarded(const sessd_pipeline_desc* desc, sessd_pipeline** out) {
     std::unique_ptr<Pipeline> P(new Pipeline());
     if (desc->frames_in_flight >= 2) {
         // R replicas, each a complete pipeline with a stream of its own; this object only holds them and the turn
@@ -499,6 +498,11 @@ int sessd_pipeline_create(const sessd_pipeline_desc* desc, sessd_pipeline** out)
     }
     *out = reinterpret_cast<sessd_pipeline*>(P.release());
     return SESSD_OK;
+}
+
+int sessd_pipeline_create(const sessd_pipeline_desc* desc, sessd_pipeline** out) {
+    if (!desc || !out) return fail(SESSD_E_INVALID, "pipeline_create: null argument");
+    return guarded(__func__, [&]() -> int { return pipeline_create_unguarded(desc, out); });
 }
 
 // the pipeline whose tensors a query is about: with frames in flight, the replica of the last submitted frame
@@ -574,7 +578,20 @@ int sessd_pipeline_join(sessd_pipeline* h, int64_t ticket, sessd_stream_t stream
     // (a ticket older than the last R frames: its replica has been reused since; waiting for the later frame on
     // it is at least as strong)
     Pipeline* rep = P->replicas[(size_t)(ticket % R)].get();
-    SESSD_HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(stream_), rep->ev_frame_done, 0));
+    // no stream to make wait: the calling thread waits (SESSD_STREAM_NONE is not a stream handle)
+    if (stream_ == SESSD_STREAM_NONE) SESSD_HIP_TRY(hipEventSynchronize(rep->ev_frame_done));
+    else SESSD_HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(stream_), rep->ev_frame_done, 0));
+    return SESSD_OK;
+}
+
+// Queries (status, layer statistics, layer tensors read back by the caller on `stream`) are about the last submitted
+// frame: with frames in flight that frame runs on its replica's own stream, which the caller's stream has to wait
+// for first.
+static int order_after_last_frame(sessd_pipeline* h, hipStream_t stream) {
+    auto* P = reinterpret_cast<Pipeline*>(h);
+    if (P->replicas.empty() || P->next_ticket == 0) return SESSD_OK;
+    Pipeline* rep = P->replicas[(size_t)P->last_replica].get();
+    SESSD_HIP_TRY(hipStreamWaitEvent(stream, rep->ev_frame_done, 0));
     return SESSD_OK;
 }
 
@@ -627,6 +644,7 @@ int sessd_pipeline_status(sessd_pipeline* h, sessd_stream_t stream_, int32_t* st
     if (!h || !status) return fail(SESSD_E_INVALID, "pipeline_status: null argument");
     Pipeline* P = current(h);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    SESSD_TRY(order_after_last_frame(h, stream));
     int32_t acc = 0, s = 0;
     SESSD_TRY(read_status_word(P->vg_ws.p, P->vg->statusOffset(P->desc.max_points), stream, &s));
     acc |= s;
@@ -646,6 +664,9 @@ int sessd_pipeline_enqueue_timed(sessd_pipeline* h, const void* points, const vo
                                  sessd_stream_t stream_, float* segment_ms, int max_segments, int* n_segments) {
     if (!h || !points || !points_size || !dense || !segment_ms || !n_segments)
         return fail(SESSD_E_INVALID, "pipeline_enqueue_timed: null argument");
+    if (!reinterpret_cast<Pipeline*>(h)->replicas.empty())
+        return fail(SESSD_E_INVALID, "pipeline_enqueue_timed: per-segment timing runs one frame on the caller's stream; "
+                                     "create the pipeline without frames_in_flight for it");
     Pipeline* P = current(h);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const int L = (int)P->stages.size();
@@ -696,6 +717,7 @@ int sessd_pipeline_layer_stats(sessd_pipeline* h, int layer, sessd_stream_t stre
     Pipeline* P = current(h);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (layer < -1 || layer >= (int)P->stages.size()) return fail(SESSD_E_INVALID, "pipeline_layer_stats: no layer %d", layer);
+    SESSD_TRY(order_after_last_frame(h, stream));
     void* num = nullptr;
     void* ws = nullptr;
     SESSD_TRY(sessd_pipeline_layer_io(h, layer, nullptr, nullptr, &num, &ws, nullptr));  // (of the same replica)

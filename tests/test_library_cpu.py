@@ -202,6 +202,20 @@ def test_creators_by_name_list_and_read_the_reference_fields():
     with pytest.raises(api.SessdError, match="has type 5, the creator reads type 1"):
         api.create_plugin("VoxelGeneratorPlugin", {"max_voxels": i32(1), "max_num_points_per_voxel": i32(5), "voxel_size": i32(1, 1, 1),
                                                    "point_cloud_range": f32(*B.POINT_CLOUD_RANGE), "voxel_feature_num": i32(4)})
+    # a vector field declared shorter than what the creator reads is refused (read out of bounds otherwise); the
+    # reference's own declaration -- length 1 on every field -- is accepted
+    with pytest.raises(api.SessdError, match="field 'point_cloud_range' declares 2 elements, the creator reads 6"):
+        api.create_plugin("VoxelGeneratorPlugin", {"max_voxels": i32(1), "max_num_points_per_voxel": i32(5), "voxel_size": f32(*B.VOXEL_SIZE),
+                                                   "point_cloud_range": f32(0, 1), "voxel_feature_num": i32(4)})
+    with pytest.raises(api.SessdError, match="field 'feature_map_size' declares 2 elements, the creator reads 3"):
+        api.create_plugin("Sparse2DensePlugin", {"feature_map_channel": i32(64), "feature_map_size": i32(176, 200)})
+    keep = [np.ascontiguousarray(v) for v in (i32(64), i32(176, 200, 2))]
+    arr = (D.PluginField * 2)()
+    for i, (k, a) in enumerate(zip((b"feature_map_channel", b"feature_map_size"), keep)):
+        arr[i].name, arr[i].data, arr[i].type, arr[i].length = k, a.ctypes.data, D.SESSD_FIELD_INT32, 1
+    h = C.c_void_p()
+    assert api.lib().sessd_plugin_create(b"Sparse2DensePlugin", C.byref(D.PluginFieldCollection(2, arr)), C.byref(h)) == 0
+    api.lib().sessd_sparse2dense_destroy(h)
     with pytest.raises(api.SessdError, match="field 'weights' is missing"):      # checked before any GPU call
         api.create_plugin("SubmConv3dLayerPlugin", {k: i32(*([3] * (3 if "shape" in k else 1))) for k in conv[:-1]})
     with pytest.raises(api.SessdError, match="holds 5 values"):
