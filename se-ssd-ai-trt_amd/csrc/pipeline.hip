@@ -117,6 +117,17 @@ struct Pipeline {
     // (voxelizer, then every layer's rulebook build in order) runs on `aux`; the GEMM chain on `stream`
     // waits per layer for the rulebook it needs, so the small build kernels of later layers overlap the
     // GEMMs of earlier ones.  Under stream capture the fork/join becomes two branches of the graph.
+    // Whether the last layer's gather-GEMM scatters into the dense tensor itself (overlapped schedule, matrix-core
+    // kernel, same element type).  The tensor is then cleared on the fill branch, beside the GEMMs, and nothing
+    // follows the last GEMM; the plugin's own cell-major pass writes fewer bytes but puts two more launches at the
+    // end of the critical path (measured: frames 20-40 us longer).
+    bool denseByEpilogue() const {
+        if (stages.empty() || !aux) return false;
+        const ConvStage& st = *stages.back();
+        const ConvPluginBase* cp = st.subm ? static_cast<const ConvPluginBase*>(st.subm.get()) : st.sparse.get();
+        return cp->out_type_ == s2d->out_type_ && cp->out_channel_ == s2d->feature_map_channel_ && cp->gemmOnMatrixCores();
+    }
+
     int enqueueOverlapped(const void* points, const void* points_size, void* dense, hipStream_t stream) {
         SESSD_HIP_TRY(hipEventRecord(ev_start, stream));
         SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_start, 0));
@@ -179,7 +190,7 @@ struct Pipeline {
                 else st->sparse->collectFill(st->ws.p, static_cast<int32_t*>(st->coors.p), f);
             }
             if (f.n + 2 > FillArgs::kMaxRegions) SESSD_TRY(flush());
-            s2d->collectFill(dense, s2d_ws.p, f);
+            if (denseByEpilogue()) s2d->collectFill(dense, s2d_ws.p, f);
             SESSD_TRY(flush());
             SESSD_HIP_TRY(hipEventRecord(ev_fill, aux_fill));
         }
@@ -219,10 +230,8 @@ struct Pipeline {
             // the last layer's epilogue also writes the dense tensor when it runs on the matrix cores and its
             // rows have the dense tensor's element type: the scatter kernel and its launch drop off the end
             // of the critical path
-            ConvPluginBase* cp = st.subm ? static_cast<ConvPluginBase*>(st.subm.get()) : st.sparse.get();
             DenseTarget dt;
-            const bool fuse = l + 1 == stages.size() && cp->out_type_ == s2d->out_type_ &&
-                              cp->out_channel_ == s2d->feature_map_channel_ && cp->gemmOnMatrixCores();
+            const bool fuse = l + 1 == stages.size() && denseByEpilogue();
             if (fuse) {
                 SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_fill, 0));
                 const int32_t* oc = st.subm ? coors : static_cast<const int32_t*>(st.coors.p);
@@ -245,7 +254,7 @@ struct Pipeline {
         SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_fill, 0));
         const void* din[3] = {feat, coors, num};
         void* dout[1] = {dense};
-        return s2d->enqueue(s2d_in, s2d_out, din, dout, s2d_ws.p, stream, true);
+        return s2d->enqueue(s2d_in, s2d_out, din, dout, s2d_ws.p, stream);
     }
 
     int enqueueDirect(const void* points, const void* points_size, void* dense, hipStream_t stream) {

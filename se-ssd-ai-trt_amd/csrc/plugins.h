@@ -219,7 +219,7 @@ class Sparse2DensePlugin {
                             const sessd_tensor_desc* outputs, int nbOutputs) const;
     int enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
                 const void* const* inputs, void* const* outputs, void* workspace,
-                hipStream_t stream, bool prefilled = false);
+                hipStream_t stream);
     void collectFill(void* dense, void* workspace, FillArgs& f) const;
     // the scatter of enqueue() as an epilogue of the gather-GEMM that produces `coors`' feature rows
     DenseTarget denseTarget(void* dense, const int32_t* coors, void* workspace) const;

@@ -547,6 +547,28 @@ def test_sparse2dense_with_folded_zero_pad():
         s2d.configure([dev(fbuf), dev(cbuf), dev(np.array([n], np.int32))], [bad])
 
 
+@pytest.mark.parametrize("size_xyz,channel,pad", [((1000, 12, 3), 40, (0, 0, 0, 0)), ((1000, 12, 3), 40, (1, 0, 3, 2)),
+                                                  ((449, 9, 1), 5, (0, 1, 0, 0)), ((7, 5, 2), 3, (0, 0, 0, 0))])
+def test_sparse2dense_long_lines_and_odd_shapes(size_xyz, channel, pad):
+    """Lines longer than one LDS segment, widths no 16-byte run divides, fewer channels than a channel group."""
+    rng = np.random.default_rng(5)
+    W, H, Dz = size_xyz
+    n, mv = min(3000, W * H * Dz // 3), 4000
+    coors = F.random_active_voxels(n, (Dz, H, W), 8)
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = rng.uniform(0.1, 1, (mv, channel)).astype(np.float32)
+    for dt in (torch.float32, torch.float16):
+        s2d = api.Sparse2Dense(size_xyz, channel, padding=pad)
+        f = dev(fbuf).to(dt)
+        dense = s2d(f, dev(cbuf), dev(np.array([n], np.int32)))
+        torch.cuda.synchronize()
+        want = O.zero_pad2d(O.sparse2dense(to_np(f[:n].float()), coors, n, size_xyz), *pad)
+        assert tuple(dense.shape) == want.shape
+        assert np.array_equal(to_np(dense.float()), want), dt
+        assert s2d.status() == 0
+
+
 def test_sparse2dense():
     rng = np.random.default_rng(2)
     n, mv, c = 2739, 60000, 64
@@ -563,6 +585,20 @@ def test_sparse2dense():
     assert dense.shape == (128, 200, 176)
     assert np.array_equal(to_np(dense), want)
     assert s2d.status() == 0
+    # the workspace may hold anything: the cell map is never cleared, a stale or random entry must not leak a row
+    ws = s2d.ws.clone()
+    for fill in (lambda t: t.fill_(0), lambda t: t.fill_(0x7f), lambda t: t.copy_(torch.randint(0, 256, t.shape, dtype=torch.uint8))):
+        fill(ws)
+        dense.fill_(3.0)
+        s2d.enqueue([dev(fbuf), dev(cbuf), dev(np.array([n], np.int32))], [dense], workspace=ws)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_np(dense), want)
+    ws32 = ws.view(torch.int32)
+    ws32.copy_(torch.randint(-3, 2 * n, ws32.shape, dtype=torch.int32))   # plausible row numbers everywhere
+    s2d.enqueue([dev(fbuf), dev(cbuf), dev(np.array([n], np.int32))], [dense], workspace=ws)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_np(dense), want)
+    assert int(ws32[0].item()) == 0
     # idempotent on a dirty output buffer, empty input gives all zeros
     dense.fill_(3.0)
     s2d.enqueue([dev(fbuf), dev(cbuf), dev(np.array([0], np.int32))], [dense])
