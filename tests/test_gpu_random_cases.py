@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import oracle_lib as O
-from gpu_util import RTOL_END_TO_END, RTOL_END_TO_END_FP16, RTOL_FP16, RTOL_FP32, assert_features_close, dev, points_input, to_np
+from gpu_util import RTOL_FP16, RTOL_FP32, abs_sum_of, assert_end_to_end_close, assert_features_close, dev, points_input, to_np
 from sessd3d import api, backbone as B, ctypes_defs as D, frames as F
 
 pytestmark = pytest.mark.gpu
@@ -56,10 +56,11 @@ def test_random_subm_layer(seed):
     what = "subm %d->%d %s n=%d grid=%s" % (cin, cout, "fp16" if half else "fp32", n, grid)
     assert conv.status() == o_st, what
     assert np.array_equal(to_np(num).astype(np.uint32), o_num), what
+    terms = abs_sum_of(feat, w, o_pairs, o_num, mv, mv, sc, sh)[:n]
     if half:
-        assert_features_close(to_np(out.float())[:n], O.round_to_half(o_out)[:n], RTOL_FP16, what)
+        assert_features_close(to_np(out.float())[:n], O.round_to_half(o_out)[:n], RTOL_FP16, what, abs_sum=terms, half=True)
     else:
-        assert_features_close(to_np(out)[:n], o_out[:n], RTOL_FP32, what)
+        assert_features_close(to_np(out)[:n], o_out[:n], RTOL_FP32, what, abs_sum=terms)
 
 
 @pytest.mark.parametrize("seed", range(30))
@@ -93,7 +94,8 @@ def test_random_strided_layer(seed):
     what = "strided k=%s s=%s p=%s in=%s %d->%d n=%d mv=%d" % (k, s, p, ig, cin, cout, n_in, mv)
     assert int(to_np(on)[0]) == o_on and conv.status() == o_st, what
     assert np.array_equal(to_np(oc), o_oc) and np.array_equal(to_np(num).astype(np.uint32), o_num), what
-    assert_features_close(to_np(out), O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), RTOL_FP32, what)
+    assert_features_close(to_np(out), O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), RTOL_FP32, what,
+                          abs_sum=abs_sum_of(feat, w, o_pairs, o_num, mv))
 
 
 def random_stack(rng):
@@ -150,5 +152,5 @@ def test_random_layer_stack_through_the_pipeline(seed):
     assert pipe.status() == ref["status"], what
     assert [pipe.layer_count(l) for l in range(-1, len(layers))] == list(ref["counts"]), what
     assert np.array_equal(pipe.read_layer(len(layers) - 1)[1], ref["coors"]), what
-    assert_features_close(to_np(dense).astype(np.float32), want, RTOL_END_TO_END_FP16 if half else RTOL_END_TO_END, what)
+    assert_end_to_end_close(to_np(dense).astype(np.float32), want, half, what)
     pipe.close()
