@@ -99,6 +99,9 @@ sp_flags(const int32_t* __restrict__ voxel_num, SpParams P, HashTable t, const u
     const uint32_t tk = blockIdx.x * kBlock + threadIdx.x;
     const int v = tk / P.Kc;
     const int n = clamp_count(voxel_num, P.max_voxels);
+    // the grid covers the capacity; a block beyond the tickets of the active rows has nothing to say, and
+    // sp_number reads no word of it
+    if ((int64_t)blockIdx.x * kBlock >= (int64_t)n * P.Kc) return;
     bool first = false;
     if (v < n) {
         const uint32_t c = cand[tk];
@@ -114,12 +117,18 @@ sp_flags(const int32_t* __restrict__ voxel_num, SpParams P, HashTable t, const u
 }
 
 __global__ void __launch_bounds__(kBlock)
-sp_number(SpParams P, HashTable t, const uint32_t* __restrict__ cand, const uint64_t* __restrict__ first_words,
-          const uint32_t* __restrict__ block_counts, int n_blocks, int32_t* __restrict__ out_coors,
-          int32_t* __restrict__ out_num, int32_t* __restrict__ nbr, int K, int32_t* meta, MirrorInit mi) {
+sp_number(const int32_t* __restrict__ voxel_num, SpParams P, HashTable t, const uint32_t* __restrict__ cand,
+          const uint64_t* __restrict__ first_words, const uint32_t* __restrict__ block_counts, int n_blocks,
+          int32_t* __restrict__ out_coors, int32_t* __restrict__ out_num, int32_t* __restrict__ nbr, int K, int32_t* meta,
+          MirrorInit mi) {
     __shared__ uint32_t lds4[4];
     const int b = blockIdx.x;
-    const int upto = b == 0 ? n_blocks : b;  // block 0 computes the total
+    // Only the blocks that hold tickets of active input rows carry anything (at a capacity of 100 000 rows and
+    // 26 000 active ones, three blocks in four would each add up thousands of counts to find nothing to number).
+    int active = (int)(((int64_t)clamp_count(voxel_num, P.max_voxels) * P.Kc + kBlock - 1) / kBlock);
+    active = active < n_blocks ? active : n_blocks;
+    if (b > 0 && b >= active) return;
+    const int upto = b == 0 ? active : b;  // block 0 computes the total
     uint32_t part = 0;
     for (int j = threadIdx.x; j < upto; j += kBlock) part += block_counts[j];
     for (int off = 32; off > 0; off >>= 1) part += __shfl_down(part, off, 64);
@@ -396,7 +405,7 @@ int SparseConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* v
     const dim3 grid(L.n_blocks), block(kBlock);
     hipLaunchKernelGGL(sp_insert, grid, block, 0, stream, coors, voxel_num, P, t, L.cand, L.meta);
     hipLaunchKernelGGL(sp_flags, grid, block, 0, stream, voxel_num, P, t, L.cand, L.first_words, L.block_counts);
-    hipLaunchKernelGGL(sp_number, grid, block, 0, stream, P, t, L.cand, L.first_words, L.block_counts,
+    hipLaunchKernelGGL(sp_number, grid, block, 0, stream, voxel_num, P, t, L.cand, L.first_words, L.block_counts,
                        L.n_blocks, out_coors, out_num, L.nbr, kernel_volume_, L.meta, mirror ? *mirror : MirrorInit());
     hipLaunchKernelGGL(sp_scatter, grid, block, 0, stream, voxel_num, P, t, L.cand, L.nbr);
     SESSD_HIP_TRY(hipGetLastError());
