@@ -62,34 +62,67 @@ __device__ __forceinline__ bool sp_candidate(const int c[3], const SpParams& P, 
     return valid;
 }
 
+// Rows that follow each other name the same output cells again and again (eight input cells share an output cell
+// of a 3x3x3 stride-2 layer, and neighbours in space are mostly neighbours in the row order), and device-wide
+// atomics are what this pass is made of.  A block therefore gathers the cells its 256 tickets name in an LDS table
+// first (cell -> smallest ticket of the block), and one thread per distinct cell goes to the table in memory.
+constexpr int kLocalBits = 9, kLocalSlots = 1 << kLocalBits;  // twice the block's tickets
+
 __global__ void __launch_bounds__(kBlock)
 sp_insert(const int32_t* __restrict__ coors, const int32_t* __restrict__ voxel_num, SpParams P, HashTable t,
           uint32_t* __restrict__ cand, int32_t* meta) {
+    __shared__ uint32_t s_key[kLocalSlots], s_val[kLocalSlots];
     const uint32_t tk = blockIdx.x * kBlock + threadIdx.x;
     const int v = tk / P.Kc, e = tk % P.Kc;
     const int n = clamp_count(voxel_num, P.max_voxels);
-    if (v >= n) return;
-    const int4 cc = reinterpret_cast<const int4*>(coors)[v];
-    const int c[3] = {cc.y, cc.z, cc.w};
-    int o[3], offset;
-    uint32_t packed = kEmpty;
-    // A negative coordinate makes the truncating divisions of getValidOutPos yield kernel offsets outside [0, K)
-    // (c = -2, k = 3, s = 2, p = 1: o = 0, offset term -1), with which the reference indexes its rulebook.  Such a
-    // row contributes nothing here and raises BAD_COORD; the offset is checked as well, so that nothing a caller
-    // passes can make sp_scatter store outside the neighbour table.
-    const bool bad = c[0] < 0 || c[1] < 0 || c[2] < 0;
-    if (bad && e == 0) atomicOr(&meta[0], SESSD_STATUS_BAD_COORD);
-    if (!bad && sp_candidate(c, P, e, o, offset) && offset >= 0 && offset < P.k[0] * P.k[1] * P.k[2]) {
-        const uint32_t key = ((uint32_t)o[0] * (uint32_t)P.os[1] + (uint32_t)o[1]) * (uint32_t)P.os[2] + (uint32_t)o[2];
+    if ((int64_t)blockIdx.x * kBlock >= (int64_t)n * P.Kc) return;  // (the whole block is beyond the active rows)
+    for (int i = threadIdx.x; i < kLocalSlots; i += kBlock) {
+        s_key[i] = kEmpty;
+        s_val[i] = kEmpty;
+    }
+    __syncthreads();
+    uint32_t key = kEmpty;
+    int offset = 0, local = -1;
+    bool owner = false;
+    if (v < n) {
+        const int4 cc = reinterpret_cast<const int4*>(coors)[v];
+        const int c[3] = {cc.y, cc.z, cc.w};
+        int o[3];
+        // A negative coordinate makes the truncating divisions of getValidOutPos yield kernel offsets outside [0, K)
+        // (c = -2, k = 3, s = 2, p = 1: o = 0, offset term -1), with which the reference indexes its rulebook.  Such a
+        // row contributes nothing here and raises BAD_COORD; the offset is checked as well, so that nothing a caller
+        // passes can make sp_scatter store outside the neighbour table.
+        const bool bad = c[0] < 0 || c[1] < 0 || c[2] < 0;
+        if (bad && e == 0) atomicOr(&meta[0], SESSD_STATUS_BAD_COORD);
+        if (!bad && sp_candidate(c, P, e, o, offset) && offset >= 0 && offset < P.k[0] * P.k[1] * P.k[2]) {
+            key = ((uint32_t)o[0] * (uint32_t)P.os[1] + (uint32_t)o[1]) * (uint32_t)P.os[2] + (uint32_t)o[2];
+            uint32_t ls = (key * 2654435769u) >> (32 - kLocalBits);
+            for (;;) {  // (at most kBlock keys in 2 * kBlock slots: room is always found)
+                const uint32_t prev = atomicCAS(&s_key[ls], kEmpty, key);
+                if (prev == kEmpty || prev == key) {
+                    owner = prev == kEmpty;
+                    break;
+                }
+                ls = (ls + 1) & (kLocalSlots - 1);
+            }
+            local = (int)ls;
+            atomicMin(&s_val[ls], tk);
+        }
+    }
+    __syncthreads();
+    if (owner) {  // this thread claimed the cell's LDS entry: it carries the block's smallest ticket to memory
         const int32_t slot = hash_insert(t, key);
         if (slot < 0) {
             atomicOr(&meta[0], SESSD_STATUS_HASH_FULL);
+            s_key[local] = kEmpty;  // (read below as "no slot")
         } else {
-            atomicMin(&t.vals[slot], tk);
-            packed = ((uint32_t)offset << kSlotBits) | (uint32_t)slot;
+            atomicMin(&t.vals[slot], s_val[local]);
+            s_val[local] = (uint32_t)slot;
         }
     }
-    cand[tk] = packed;
+    __syncthreads();
+    if (v >= n) return;
+    cand[tk] = (local >= 0 && s_key[local] != kEmpty) ? (((uint32_t)offset << kSlotBits) | s_val[local]) : kEmpty;
 }
 
 __global__ void __launch_bounds__(kBlock)
