@@ -166,14 +166,28 @@ struct Pipeline {
                 }
             }
         }
-        // The voxelizer heads the frame's critical path: it is queued (and, in a graph, submitted) before
-        // anything else.
+        // The head of the frame -- the voxelizer and the lookups of the SubM layers on its voxels, which the first
+        // GEMMs wait for -- runs on the caller's stream itself, in front of those GEMMs: a kernel starts 1-2 us
+        // behind its producer on the same branch of the graph and 5-10 us behind one on another branch.  The
+        // status words of those SubM layers are cleared in the voxelizer's own clear launch.
+        const bool head_off = false;
+        std::vector<char> on_head(stages.size(), 0);
+        FillArgs head_clears;
+        for (size_t l = 0; l < stages.size() && !head_off; ++l) {
+            ConvStage& st = *stages[l];
+            if (!st.subm) break;
+            if (st.rulebook_from >= 0) continue;
+            if (!probes_upstream[l] || !st.ws.p) break;
+            on_head[l] = 1;
+            st.subm->collectFill(st.ws.p, head_clears, false);
+        }
+        hipStream_t head = head_off ? aux : stream;
         const void* vin[2] = {points, points_size};
         void* vout[3] = {vg_voxels.p, vg_coors.p, vg_num.p};
-        SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, aux, mirror_of[0].nbr ? &mirror_of[0] : nullptr));
-        SESSD_HIP_TRY(hipEventRecord(ev_vg, aux));
+        SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, head, mirror_of[0].nbr ? &mirror_of[0] : nullptr, &head_clears));
+        SESSD_HIP_TRY(hipEventRecord(ev_vg, head));
         SESSD_HIP_TRY(hipStreamWaitEvent(aux_fill, ev_start, 0));
-        // every clear of the frame (hash tables, neighbour tables, status words, the dense tensor) has no
+        // every other clear of the frame (hash tables, neighbour tables, status words, the dense tensor) has no
         // input: they run batched on a third stream while the voxelizer works
         {
             FillArgs f;
@@ -184,7 +198,7 @@ struct Pipeline {
             };
             for (size_t l = 0; l < stages.size(); ++l) {
                 auto& st = stages[l];
-                if (!st->ws.p) continue;
+                if (!st->ws.p || on_head[l]) continue;
                 if (f.n + 6 > FillArgs::kMaxRegions) SESSD_TRY(flush());
                 if (st->subm) st->subm->collectFill(st->ws.p, f, !probes_upstream[l]);
                 else st->sparse->collectFill(st->ws.p, static_cast<int32_t*>(st->coors.p), f);
@@ -194,6 +208,7 @@ struct Pipeline {
             SESSD_TRY(flush());
             SESSD_HIP_TRY(hipEventRecord(ev_fill, aux_fill));
         }
+        if (!head_off) SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_vg, 0));
         SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_fill, 0));
         const int32_t* coors = static_cast<const int32_t*>(vg_coors.p);
         const int32_t* num = static_cast<const int32_t*>(vg_num.p);
@@ -202,8 +217,9 @@ struct Pipeline {
             ConvStage& st = *stages[l];
             if (st.subm) {
                 if (st.rulebook_from >= 0) continue;
-                SESSD_TRY(st.subm->enqueueBuild(coors, num, st.ws.p, aux, true, probes_upstream[l] ? &cells : nullptr,
-                                                mirrored[l] != 0));
+                SESSD_TRY(st.subm->enqueueBuild(coors, num, st.ws.p, on_head[l] ? stream : aux, true,
+                                                probes_upstream[l] ? &cells : nullptr, mirrored[l] != 0));
+                if (on_head[l]) continue;  // (its GEMM follows on the same stream: no event)
             } else {
                 SESSD_TRY(st.sparse->enqueueBuild(coors, num, static_cast<int32_t*>(st.coors.p),
                                                   static_cast<int32_t*>(st.num.p), st.ws.p, aux, true,
@@ -214,7 +230,7 @@ struct Pipeline {
             }
             SESSD_HIP_TRY(hipEventRecord(ev_build[l], aux));
         }
-        SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_vg, 0));
+        if (head_off) SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_vg, 0));
         const void* feat = vg_voxels.p;
         coors = static_cast<const int32_t*>(vg_coors.p);
         num = static_cast<const int32_t*>(vg_num.p);
@@ -224,7 +240,7 @@ struct Pipeline {
             ConvStage& st = *stages[l];
             const int owner = st.rulebook_from >= 0 ? st.rulebook_from : (int)l;
             if (owner > last_waited) {
-                SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_build[owner], 0));
+                if (!on_head[(size_t)owner]) SESSD_HIP_TRY(hipStreamWaitEvent(stream, ev_build[owner], 0));
                 last_waited = owner;
             }
             // the last layer's epilogue also writes the dense tensor when it runs on the matrix cores and its

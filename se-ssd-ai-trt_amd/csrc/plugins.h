@@ -28,10 +28,11 @@ class VoxelGeneratorPlugin {
                         int nbOutputs);
     size_t getWorkspaceSize(const sessd_tensor_desc* inputs, int nbInputs,
                             const sessd_tensor_desc* outputs, int nbOutputs) const;
-    // `mirror`: the neighbour table of the SubM layer that will run its symmetric lookup on these voxels
+    // `mirror`: the neighbour table of the SubM layer that will run its symmetric lookup on these voxels;
+    // `also_clear`: regions cleared in the same launch as the voxelizer's own tables
     int enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,
                 const void* const* inputs, void* const* outputs, void* workspace,
-                hipStream_t stream, const MirrorInit* mirror = nullptr);
+                hipStream_t stream, const MirrorInit* mirror = nullptr, const FillArgs* also_clear = nullptr);
     // enqueue() on the library's own static scratch array instead of a caller's workspace: allocates nothing;
     // rejects points tensors whose layout does not fit the array.  Calls that overlap on one GPU race.
     int enqueueStatic(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc* outputDesc,

@@ -327,7 +327,7 @@ size_t VoxelGeneratorPlugin::statusOffset(int max_points) const {
 
 int VoxelGeneratorPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sessd_tensor_desc*,
                                   const void* const* inputs, void* const* outputs, void* workspace,
-                                  hipStream_t stream, const MirrorInit* mirror) {
+                                  hipStream_t stream, const MirrorInit* mirror, const FillArgs* also_clear) {
     if (!inputDesc || !inputs || !outputs || !workspace)
         return fail(SESSD_E_INVALID, "voxelgen.enqueue: null argument");
     if (inputDesc[0].nbDims != 3 || inputDesc[0].d[0] != 1)
@@ -360,6 +360,10 @@ int VoxelGeneratorPlugin::enqueue(const sessd_tensor_desc* inputDesc, const sess
     if (!(flags_ & SESSD_FLAG_SKIP_PAD_ROWS)) {  // voxelGenerator.cu:524-525
         f.add(voxels, (uint64_t)voxelNum_ * 4, 0);
         f.add(coors, (uint64_t)voxelNum_ * 4, 0);
+    }
+    if (also_clear) {  // a pipeline's small clears ride along in the launch that heads the frame anyway
+        if (f.n + also_clear->n > FillArgs::kMaxRegions) return fail(SESSD_E_INVALID, "voxelgen.enqueue: too many regions to clear");
+        for (int i = 0; i < also_clear->n; ++i) f.r[f.n++] = also_clear->r[i];
     }
     SESSD_TRY(launch_fill(f, stream));
 
