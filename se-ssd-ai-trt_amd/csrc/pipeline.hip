@@ -88,9 +88,9 @@ struct Pipeline {
     int64_t next_ticket = 0;
     int last_replica = 0;                       // replica of the last submitted frame (layer_io, status, stats)
 
-    // two-stream schedule: coordinate chain (voxelizer + rulebook builds) on `aux`, feature chain on the
-    // caller's stream; ev_build[l] = "rulebook of layer l is ready"
-    hipStream_t aux = nullptr, aux_fill = nullptr;
+    // two-stream schedule: the frame's clears and the rulebook builds on `aux`; the voxelizer, the lookups on its
+    // voxels and the feature chain on the caller's stream; ev_build[l] = "rulebook of layer l is ready"
+    hipStream_t aux = nullptr;
     hipEvent_t ev_start = nullptr, ev_vg = nullptr, ev_fill = nullptr;
     std::vector<hipEvent_t> ev_build;
 
@@ -110,7 +110,6 @@ struct Pipeline {
         if (ev_vg) (void)hipEventDestroy(ev_vg);
         if (ev_fill) (void)hipEventDestroy(ev_fill);
         if (aux) (void)hipStreamDestroy(aux);
-        if (aux_fill) (void)hipStreamDestroy(aux_fill);
     }
 
     // The rulebooks depend only on coordinates, the GEMMs on rulebooks + features.  The coordinate chain
@@ -186,13 +185,13 @@ struct Pipeline {
         void* vout[3] = {vg_voxels.p, vg_coors.p, vg_num.p};
         SESSD_TRY(vg->enqueue(vg_in, vg_out, vin, vout, vg_ws.p, head, mirror_of[0].nbr ? &mirror_of[0] : nullptr, &head_clears));
         SESSD_HIP_TRY(hipEventRecord(ev_vg, head));
-        SESSD_HIP_TRY(hipStreamWaitEvent(aux_fill, ev_start, 0));
         // every other clear of the frame (hash tables, neighbour tables, status words, the dense tensor) has no
-        // input: they run batched on a third stream while the voxelizer works
+        // input: they run batched at the head of `aux`, which has nothing else to do while the voxelizer works (a
+        // stream of their own measured the same)
         {
             FillArgs f;
             auto flush = [&]() -> int {
-                const int rc = launch_fill(f, aux_fill);
+                const int rc = launch_fill(f, aux);
                 f = FillArgs();
                 return rc;
             };
@@ -206,10 +205,9 @@ struct Pipeline {
             if (f.n + 2 > FillArgs::kMaxRegions) SESSD_TRY(flush());
             if (denseByEpilogue()) s2d->collectFill(dense, s2d_ws.p, f);
             SESSD_TRY(flush());
-            SESSD_HIP_TRY(hipEventRecord(ev_fill, aux_fill));
+            SESSD_HIP_TRY(hipEventRecord(ev_fill, aux));
         }
         if (!head_off) SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_vg, 0));
-        SESSD_HIP_TRY(hipStreamWaitEvent(aux, ev_fill, 0));
         const int32_t* coors = static_cast<const int32_t*>(vg_coors.p);
         const int32_t* num = static_cast<const int32_t*>(vg_num.p);
         HashTable cells = vg->cellTable(vg_ws.p, desc.max_points);  // the table upstream of the current layer
@@ -436,7 +434,6 @@ static int build_pipeline(const sessd_pipeline_desc& d, Pipeline* P) {
     P->device_bytes = total;
     if (d.overlap_streams) {
         SESSD_HIP_TRY(hipStreamCreateWithFlags(&P->aux, hipStreamNonBlocking));
-        SESSD_HIP_TRY(hipStreamCreateWithFlags(&P->aux_fill, hipStreamNonBlocking));
         SESSD_HIP_TRY(hipEventCreateWithFlags(&P->ev_fill, hipEventDisableTiming));
         SESSD_HIP_TRY(hipEventCreateWithFlags(&P->ev_start, hipEventDisableTiming));
         SESSD_HIP_TRY(hipEventCreateWithFlags(&P->ev_vg, hipEventDisableTiming));
