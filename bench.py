@@ -382,9 +382,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-parity", action="store_true", help="skip the comparison with the CPU oracle")
     ap.add_argument("--no-others", action="store_true", help="only the headline configuration")
-    ap.add_argument("--frames-in-flight", type=int, default=3,
+    ap.add_argument("--frames-in-flight", type=int, default=2,
                     help="replicas of the pipeline for the throughput figure with frames in flight (sessd_pipeline_submit / "
-                         "join); 3 measured best with HIP's default of 4 hardware queues; 0 = skip")
+                         "join); a replica runs on two streams and HIP has 4 hardware queues by default: 2 and 4 replicas "
+                         "measured best, 3 worse than one frame at a time; 0 = skip")
     ap.add_argument("--config5-frames", type=int, default=100,
                     help="seeded frames of configuration 5 in other_configs (its stated repetition is 100; a pool of "
                          "threads generates them, ~0.1 s a frame)")
