@@ -297,10 +297,12 @@ int sessd_sparse2dense_serialize(const sessd_sparse2dense* h, void* buf);
 /* replaces configurePlugin (sparse2Dense.cu:170-173) */
 int sessd_sparse2dense_configure(sessd_sparse2dense* h, const sessd_tensor_desc* in, int nIn,
                                  const sessd_tensor_desc* out, int nOut);
-/* replaces getWorkspaceSize (sparse2Dense.cu:175-179); only the status word */
+/* replaces getWorkspaceSize (sparse2Dense.cu:175-179: the reference needs none); here the status word, one word per
+ * 256 rows and a cell -> row map of D*H*W ints (282 KB for 2 x 200 x 176) */
 size_t sessd_sparse2dense_workspace_size(const sessd_sparse2dense* h, const sessd_tensor_desc* in,
                                          int nIn, const sessd_tensor_desc* out, int nOut);
-/* replaces enqueue (sparse2Dense.cu:224-249); workspace may be NULL */
+/* replaces enqueue (sparse2Dense.cu:224-249).  The workspace is required (SESSD_E_INVALID when NULL); its contents
+ * need not be cleared or kept between calls.  Every element of the output is written, zeros included. */
 int sessd_sparse2dense_enqueue(sessd_sparse2dense* h, const sessd_tensor_desc* inDesc,
                                const sessd_tensor_desc* outDesc, const void* const* inputs,
                                void* const* outputs, void* workspace, sessd_stream_t stream);
