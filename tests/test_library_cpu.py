@@ -150,6 +150,16 @@ def test_sparse2dense_host_side():
     assert struct.unpack("<4i", blob[:16]) == (176, 200, 2, 64) and struct.unpack("<4i", blob[20:]) == (1, 2, 3, 4)
     assert api.Sparse2Dense.deserialize(blob).serialize() == blob
     assert L.sessd_sparse2dense_set_padding(p.h, -1, 0, 0, 0) == D.SESSD_E_INVALID
+    # the workspace: status block, one word per 256 rows, the cell -> row map; an enqueue without one is refused
+    # before any runtime call (the reference's plugin needs none, sparse2Dense.cu:175-179)
+    ind = (D.TensorDesc * 3)(D.TensorDesc.make([1, 60000, 64], D.SESSD_FLOAT), D.TensorDesc.make([1, 60000, 4], D.SESSD_INT32),
+                             D.TensorDesc.make([1], D.SESSD_INT32))
+    outd = (D.TensorDesc * 1)(D.TensorDesc.make([1, 128, 200, 176], D.SESSD_FLOAT))
+    assert L.sessd_sparse2dense_configure(s.h, ind, 3, outd, 1) == D.SESSD_OK
+    assert L.sessd_sparse2dense_workspace_size(s.h, ind, 3, outd, 1) == 256 + 1024 + 2 * 200 * 176 * 4
+    fake = (C.c_void_p * 3)(4096, 8192, 12288)                # never dereferenced: the call fails first
+    assert L.sessd_sparse2dense_enqueue(s.h, ind, outd, fake, fake, None, None) == D.SESSD_E_INVALID
+    assert b"workspace" in L.sessd_last_error()
 
 
 def test_conv_create_validates_before_touching_the_gpu():
