@@ -195,10 +195,15 @@ export_pairs(const int32_t* __restrict__ nbr, int max_voxels, int words_per_k,
 int launch_mfma(const GemmArgs& a, hipStream_t stream);  // conv_mfma.hip
 
 int launch_tall(const GemmArgs& a, hipStream_t stream);  // conv_tall.hip
+int launch_wide(const GemmArgs& a, hipStream_t stream);  // conv_wide.hip
 
 int launch_gather_gemm(const GemmArgs& a, hipStream_t stream) {
     if (!a.force_valu) {  // FP16 3x3x3 layers from 32 channels up: the tall-tile kernel
         const int rc = launch_tall(a, stream);
+        if (rc != SESSD_E_UNSUPPORTED) return rc;
+    }
+    if (!a.force_valu) {  // FP32 64 -> 64: one tall tile per compute unit
+        const int rc = launch_wide(a, stream);
         if (rc != SESSD_E_UNSUPPORTED) return rc;
     }
     if (!a.force_valu) {

@@ -524,7 +524,10 @@ void chunk_shape(int dtype, int cin, int* channels, int* lane_elems) {
 
 int gemm_compute_units() { return compute_units(); }
 
-int gemm_tile_rows(int cin, int cout, int dtype) { return tile_rows(dtype == SESSD_HALF && cin != 4, cin, cout); }
+int gemm_tile_rows(int cin, int cout, int dtype) {
+    if (gemm_runs_wide(kMaxK, cin, cout, dtype, dtype)) return gemm_wide_tile_rows();
+    return tile_rows(dtype == SESSD_HALF && cin != 4, cin, cout);
+}
 
 bool gemm_runs_on_mfma(int K, int cin, int cout, int in_type, int out_type) {
     if (!mfma_shape(K, cin, cout, out_type)) return false;

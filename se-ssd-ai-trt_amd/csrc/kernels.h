@@ -68,6 +68,10 @@ bool gemm_runs_on_mfma(int K, int cin, int cout, int in_type, int out_type);
 // whether the layer runs on the tall-tile FP16 kernel (conv_tall.hip), which cuts its own tiles: a rulebook whose
 // owner does needs no equal-work cuts
 bool gemm_runs_tall(int K, int cin, int cout, int in_type, int out_type);
+// whether the layer runs on the FP32 kernel with one tall tile per compute unit (conv_wide.hip), and that kernel's
+// tile capacity
+bool gemm_runs_wide(int K, int cin, int cout, int in_type, int out_type);
+int gemm_wide_tile_rows();
 
 // size in bytes of the packed weight copy for this shape/dtype (0 = shape runs on the VALU path)
 size_t packed_weight_bytes(int K, int cin, int cout, int dtype);
