@@ -51,7 +51,7 @@ def kernel_source_hash():
     """Short hash of the gather-GEMM kernels' sources: the committed counter summaries carry the hash of the sources
     they were collected on, so a figure taken from them can be told from a stale one."""
     h = hashlib.sha256()
-    for name in ("conv_mfma.hip", "conv_tall.hip"):
+    for name in ("conv_mfma.hip", "conv_tall.hip", "conv_wide.hip"):
         with open(os.path.join(ROOT, "se-ssd-ai-trt_amd", "csrc", name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:12]
@@ -315,8 +315,9 @@ def measure(config, args, torch, frames=None, points_override=None, deep=True, w
         ach = dom_bytes / (dom_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None}
-    # (FP16 3x3x3 layers from 32 channels up run on the tall-tile kernel, everything else on the split-K one)
-    kname = ("conv_tall<%d, %d," if half else "conv_mfma<float, %d, %d,") % (dom_c, dom_c)
+    # (FP16 3x3x3 layers from 32 channels up run on the tall-tile kernel, FP32 64 -> 64 on the one-tile-per-unit
+    # kernel, everything else on the split-K one)
+    kname = ("conv_tall<%d, %d," if half else "conv_wide<%d, %d>" if dom_c == 64 else "conv_mfma<float, %d, %d,") % (dom_c, dom_c)
     traffic, fresh = profiled_traffic(kname, config, dtype)
     roof["traffic"] = traffic
     roof.update({"traffic_source": "profiles/frame_pipeline_config%d_%s.md (rocprofv3 FETCH_SIZE/WRITE_SIZE), collected on %s"
