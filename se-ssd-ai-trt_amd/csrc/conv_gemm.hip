@@ -202,7 +202,7 @@ int launch_gather_gemm(const GemmArgs& a, hipStream_t stream) {
         const int rc = launch_tall(a, stream);
         if (rc != SESSD_E_UNSUPPORTED) return rc;
     }
-    if (!a.force_valu) {  // FP32 64 -> 64: one tall tile per compute unit
+    if (!a.force_valu) {  // FP32, 64 output columns: one tall tile per compute unit
         const int rc = launch_wide(a, stream);
         if (rc != SESSD_E_UNSUPPORTED) return rc;
     }

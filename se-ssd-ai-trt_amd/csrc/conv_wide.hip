@@ -1,4 +1,5 @@
-// conv_wide.hip -- FP32 gather-GEMM for the wide layers: one tall tile per compute unit, sixteen waves.
+// conv_wide.hip -- FP32 gather-GEMM for the layers with 64 output columns (Cin 32 or 64): one tall tile per compute
+// unit, sixteen waves.
 //
 //     out[o][:] = epilogue( sum_k  in[nbr[k][o]][:] @ W[k] )
 //
@@ -25,9 +26,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned int v4u32 __attribute__((__vector_size__(16)));
 
 constexpr int kWaves = 16;          // wave64s per workgroup: four per SIMD
-constexpr int kCS = 4;              // waves of a group (column quarters)
-constexpr int kKG = kWaves / kCS;   // groups the offsets are dealt to
-constexpr int kTileRows = 96;       // tile capacity (rows)
+constexpr int kTileRows = 96;       // tile capacity (rows): what the partial tiles leave of the 160 KB of LDS
 constexpr int kMaxBlk = kTileRows / 16;
 constexpr int kMaxK = kGemmMaxOffsets;
 constexpr unsigned kOutOfRange = 0x80000000u;  // beyond any buffer the kernel is given (launch() checks)
@@ -53,9 +52,12 @@ conv_wide(const float* __restrict__ in, float* __restrict__ out, const void* __r
           const int32_t* __restrict__ tiles, DenseTarget dt) {
     constexpr int G = CIN / 16;     // 16-channel chunks of the inner dimension
     constexpr int NBT = COUT / 16;  // 16-column blocks of the layer
-    constexpr int NB = NBT / kCS;   // ... of one wave
+    constexpr int kCS = 4;               // waves of a group (column quarters)
+    constexpr int kKG = kWaves / kCS;    // groups the offsets are dealt to
+    constexpr int NB = NBT / kCS;   // column blocks of one wave
     constexpr int CW = COUT / kCS;  // columns of one wave
     constexpr int LDP = CW + 4;     // padded row stride of a partial tile
+    static_assert(kTileRows <= 128 && kTileRows % 16 == 0, "the lists are staged in two halves of 64 rows");
     constexpr int kVecPerRow = COUT / 4;
     constexpr int kThreads = kWaves * 64;
     static_assert(CIN % 16 == 0 && NBT % kCS == 0, "channel counts must fill whole MFMA chunks per wave");
@@ -338,7 +340,7 @@ int launch(const GemmArgs& a, hipStream_t stream) {
 
 bool gemm_runs_wide(int K, int cin, int cout, int in_type, int out_type) {
     if (in_type != SESSD_FLOAT || out_type != SESSD_FLOAT || K > kMaxK) return false;
-    return cin == 64 && cout == 64;
+    return cout == 64 && (cin == 64 || cin == 32);
 }
 
 int gemm_wide_tile_rows() { return kTileRows; }
@@ -347,6 +349,7 @@ int launch_wide(const GemmArgs& a, hipStream_t stream) {
     if (!a.w_packed || !gemm_runs_wide(a.K, a.cin, a.cout, a.in_type, a.out_type)) return SESSD_E_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(a.in_feat) | reinterpret_cast<uintptr_t>(a.out_feat)) & 15) return SESSD_E_UNSUPPORTED;
     if (a.cin == 64 && a.cout == 64) return launch<64, 64>(a, stream);
+    if (a.cin == 32 && a.cout == 64) return launch<32, 64>(a, stream);
     return SESSD_E_UNSUPPORTED;
 }
 

@@ -745,14 +745,14 @@ def test_tall_fp16_kernel_with_two_row_blocks_per_wave(cin, cout, n):
 
 
 # ---------------------------------------------------------------------------------------------
-# the FP32 64 -> 64 kernel with one tall tile per compute unit (conv_wide.hip)
+# the FP32 kernel with one tall tile per compute unit (conv_wide.hip: 64 -> 64 and 32 -> 64)
 # ---------------------------------------------------------------------------------------------
-def _fp32_subm_64_against_oracle(n, mv, grid, seed, clustered=True, epilogue=True, threads=1):
+def _fp32_subm_wide_against_oracle(n, mv, grid, seed, clustered=True, epilogue=True, threads=1, cin=64):
     rng = np.random.default_rng(seed)
     coors = (F.clustered_active_voxels(n, grid, seed, n_blobs=max(4, n // 100)) if clustered
              else F.random_active_voxels(n, grid, seed))
-    feat = rng.uniform(-1, 1, (n, 64)).astype(np.float32)
-    w = rng.normal(0, 0.1, (27, 64, 64)).astype(np.float32)
+    feat = rng.uniform(-1, 1, (n, cin)).astype(np.float32)
+    w = rng.normal(0, 0.1, (27, cin, 64)).astype(np.float32)
     sc = rng.uniform(0.5, 1.5, 64).astype(np.float32) if epilogue else None
     sh = rng.uniform(-0.2, 0.2, 64).astype(np.float32) if epilogue else None
     conv, out, pairs, num, cbuf = run_subm(coors, n, feat, w, grid, mv, sc, sh, epilogue)
@@ -766,24 +766,25 @@ def _fp32_subm_64_against_oracle(n, mv, grid, seed, clustered=True, epilogue=Tru
     if epilogue:
         o_out = O.scale_shift_relu(o_out, mv, sc, sh, True)
     # every row of the tensor: rows >= n are the epilogue of zero (the reference zero-fills, then BN + ReLU)
-    assert_features_close(out, o_out, RTOL_FP32, "wide fp32 64->64, %d rows" % n,
+    assert_features_close(out, o_out, RTOL_FP32, "wide fp32 %d->64, %d rows" % (cin, n),
                           abs_sum=abs_sum_of(feat, w, o_pairs, o_num, mv, mv, sc, sh))
     assert conv.status() == 0
     conv.close()
 
 
+@pytest.mark.parametrize("cin", [64, 32])
 @pytest.mark.parametrize("n", [1, 15, 16, 17, 63, 64, 65, 95, 96, 97, 255, 256, 257, 1000])
-def test_wide_fp32_kernel_row_counts_around_its_tiles(n):
+def test_wide_fp32_kernel_row_counts_around_its_tiles(n, cin):
     """One workgroup per compute unit walks tiles of up to 96 rows whose neighbour lists are staged in two halves
     of 64 rows: row counts on either side of a 16-pair block, the staging halves, the tile capacity and the number
     of compute units (256 rows: one row per tile), against the oracle (pad rows included)."""
-    _fp32_subm_64_against_oracle(n, n + 200, (5, 40, 40), 700 + n, epilogue=(n % 2 == 1))
+    _fp32_subm_wide_against_oracle(n, n + 200, (5, 40, 40), 700 + n, epilogue=(n % 2 == 1), cin=cin)
 
 
-@pytest.mark.parametrize("n,clustered", [(20000, True), (24577, False), (50000, True)])
-def test_wide_fp32_kernel_tall_tiles_and_two_tiles_per_workgroup(n, clustered):
+@pytest.mark.parametrize("n,clustered,cin", [(20000, True, 64), (20000, True, 32), (24577, False, 64), (50000, True, 64)])
+def test_wide_fp32_kernel_tall_tiles_and_two_tiles_per_workgroup(n, clustered, cin):
     """~78-row tiles (20 000 rows: both staging halves in use), the first row count past one 96-row tile per
     compute unit (24 577 rows of scattered voxels: every workgroup walks two tiles), and 50 000 clustered rows
     (tiles of uneven length from the equal-work cuts, two or three per workgroup), against the oracle on 16
     threads."""
-    _fp32_subm_64_against_oracle(n, 51200, (21, 400, 352), 5000 + n, clustered=clustered, threads=16)
+    _fp32_subm_wide_against_oracle(n, 51200, (21, 400, 352), 5000 + n, clustered=clustered, threads=16, cin=cin)
