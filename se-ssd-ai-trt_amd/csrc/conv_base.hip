@@ -101,6 +101,9 @@ bool ConvPluginBase::gemmOnMatrixCores() const {
 }
 
 int ConvPluginBase::tileRows() const { return gemm_tile_rows(in_channel_, out_channel_, out_type_); }
+int ConvPluginBase::tileRowWeight() const {
+    return gemm_runs_wide(kernel_volume_, in_channel_, out_channel_, in_type_, out_type_) ? 4 : 20;
+}
 
 int ConvPluginBase::runGemm(const void* in_feat, void* out_feat, const int32_t* nbr, const int32_t* tiles,
                             const int32_t* num_out, hipStream_t stream, const DenseTarget* dense) {

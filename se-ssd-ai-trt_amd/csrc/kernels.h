@@ -58,7 +58,7 @@ int gemm_compute_units();
 // workspace; its first word must be zero before the launch and stays zero when there are no active rows);
 // target_rows >= kGemmMinTileRows is the tile height aimed at
 size_t tile_cut_bytes(int max_voxels);
-int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, int target_rows,
+int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, int target_rows, int row_weight,
                      void* region, hipStream_t stream);
 
 // picks the kernel for the layer shape; returns SESSD_E_UNSUPPORTED for dtype pairs not covered, and when a

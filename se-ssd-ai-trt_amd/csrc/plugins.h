@@ -114,6 +114,8 @@ class ConvPluginBase {
     }
     // tile height those cuts aim at: the capacity of this layer's own GEMM kernel
     int tileRows() const;
+    // weight of a row beside its pairs in those cuts
+    int tileRowWeight() const;
     int exportRulebook(const int32_t* nbr, const int32_t* num_out, void* scratch,
                        int32_t* indice_pairs, uint32_t* indice_num, hipStream_t stream) const;
     int freeDevice();

@@ -442,7 +442,7 @@ int SparseConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* v
                        L.n_blocks, out_coors, out_num, L.nbr, kernel_volume_, L.meta, mirror ? *mirror : MirrorInit());
     hipLaunchKernelGGL(sp_scatter, grid, block, 0, stream, voxel_num, P, t, L.cand, L.nbr);
     SESSD_HIP_TRY(hipGetLastError());
-    if (wantTileCuts()) SESSD_TRY(launch_tile_cuts(L.nbr, out_num, kernel_volume_, max_voxels_, tileRows(), L.tiles, stream));
+    if (wantTileCuts()) SESSD_TRY(launch_tile_cuts(L.nbr, out_num, kernel_volume_, max_voxels_, tileRows(), tileRowWeight(), L.tiles, stream));
     return SESSD_OK;
 }
 

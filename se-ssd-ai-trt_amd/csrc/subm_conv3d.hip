@@ -285,7 +285,7 @@ int SubmConv3dLayerPlugin::enqueueBuild(const int32_t* coors, const int32_t* vox
                            voxel_num, max_voxels_, g, ksize_, padding_, cells ? *cells : t, L.nbr,
                            cells ? L.meta : nullptr);
     SESSD_HIP_TRY(hipGetLastError());
-    if (wantTileCuts()) SESSD_TRY(launch_tile_cuts(L.nbr, voxel_num, kernel_volume_, max_voxels_, tileRows(), L.tiles, stream));
+    if (wantTileCuts()) SESSD_TRY(launch_tile_cuts(L.nbr, voxel_num, kernel_volume_, max_voxels_, tileRows(), tileRowWeight(), L.tiles, stream));
     return SESSD_OK;
 }
 

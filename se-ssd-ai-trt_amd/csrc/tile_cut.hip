@@ -4,10 +4,13 @@
 // The GEMM kernel gives every workgroup a run of consecutive output rows.  With runs of equal length the
 // busiest compute unit of the headline frame issues 37 % more MFMA blocks than the average one (pairs per
 // row vary between 1 and 27 with the local density of the scene), and the launch lasts as long as the
-// busiest unit.  Here every row gets the weight  pairs(row) + kRowWeight  and the rows are cut where the
+// busiest unit.  Here every row gets the weight  pairs(row) + row_weight  and the rows are cut where the
 // running sum crosses multiples of W = ceil(total / T), T = the tile count the equal-length rule would
-// use (tile_plan() with the target height the caller names).  The constant keeps sparse runs from growing far beyond the kernel's tile capacity;
-// runs that still do are walked in capacity-sized pieces by the kernel, so any cut is correct.
+// use (tile_plan() with the target height the caller names).  The per-row constant is the caller's: what a row
+// costs its GEMM kernel beside its pairs (20 pairs' worth on the split-K kernel, 4 on the one-tile-per-unit kernel,
+// whose tile time measured 732 cycles per 16-pair block + 22 per row); it also keeps sparse runs from growing far
+// beyond the kernel's tile capacity.  Runs that still do are walked in capacity-sized pieces by the kernel, so any
+// cut is correct.
 //
 // Two launches over the rows:
 //   tile_weights  row weight -> w[row], per-block sums -> bsum[block]
@@ -23,7 +26,6 @@ namespace sessd {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kRowWeight = 20;  // fixed cost of a row beside its pairs
 
 __host__ __device__ inline int max_tiles(int max_voxels) { return max_voxels / kGemmMinTileRows + 1024 + 1; }
 
@@ -31,7 +33,7 @@ __host__ __device__ inline int max_tiles(int max_voxels) { return max_voxels / k
 constexpr int kSplit = 4;
 __global__ void __launch_bounds__(kBlock * kSplit)
 tile_weights(const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
-             int32_t* __restrict__ w, int32_t* __restrict__ bsum) {
+             int row_weight, int32_t* __restrict__ w, int32_t* __restrict__ bsum) {
     __shared__ int32_t s_cnt[kSplit][kBlock];
     __shared__ int32_t s_part[kBlock / 64];
     int n = *num_out;
@@ -54,7 +56,7 @@ tile_weights(const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_ou
     __syncthreads();
     int v = 0;
     if (kg == 0 && row < n) {
-        v = kRowWeight;
+        v = row_weight;
 #pragma unroll
         for (int g = 0; g < kSplit; ++g) v += s_cnt[g][r];
     }
@@ -68,7 +70,7 @@ tile_weights(const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_ou
 }
 
 __global__ void __launch_bounds__(kBlock)
-tile_cuts(const int32_t* __restrict__ num_out, int max_voxels, int num_cu, int target, const int32_t* __restrict__ w,
+tile_cuts(const int32_t* __restrict__ num_out, int max_voxels, int num_cu, int target, int row_weight, const int32_t* __restrict__ w,
           const int32_t* __restrict__ bsum, int32_t* __restrict__ hdr) {
     __shared__ int32_t s_before[kBlock / 64], s_total[kBlock / 64], s_wave[kBlock / 64];
     int n = *num_out;
@@ -113,7 +115,7 @@ tile_cuts(const int32_t* __restrict__ num_out, int max_voxels, int num_cu, int t
     // up to the last gets its start written (with few rows -- fewer than tiles -- total / tiles would fall
     // below a row's weight, ids would skip, and the skipped entries of the table would be read unwritten)
     int W = (total + tiles - 1) / tiles;
-    W = W > kGemmMaxOffsets + kRowWeight ? W : kGemmMaxOffsets + kRowWeight + 1;
+    W = W > kGemmMaxOffsets + row_weight ? W : kGemmMaxOffsets + row_weight + 1;
     if (row < n) {
         const int id = excl / W;
         const int prev = row == 0 ? -1 : (excl - w[row - 1]) / W;
@@ -135,15 +137,15 @@ size_t tile_cut_bytes(int max_voxels) {
     return align_up(ints * sizeof(int32_t));
 }
 
-int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, int target_rows,
+int launch_tile_cuts(const int32_t* nbr, const int32_t* num_out, int K, int max_voxels, int target_rows, int row_weight,
                      void* region, hipStream_t stream) {
     if (target_rows < kGemmMinTileRows) return fail(SESSD_E_INVALID, "tile cuts: target of %d rows is below %d", target_rows, kGemmMinTileRows);
     int32_t* hdr = static_cast<int32_t*>(region);
     int32_t* w = hdr + 4 + max_tiles(max_voxels) + 1;
     int32_t* bsum = w + max_voxels;
     const int blocks = ceil_div(max_voxels, kBlock);
-    hipLaunchKernelGGL(tile_weights, dim3(blocks), dim3(kBlock * kSplit), 0, stream, nbr, num_out, max_voxels, K, w, bsum);
-    hipLaunchKernelGGL(tile_cuts, dim3(blocks), dim3(kBlock), 0, stream, num_out, max_voxels, gemm_compute_units(), target_rows, w,
+    hipLaunchKernelGGL(tile_weights, dim3(blocks), dim3(kBlock * kSplit), 0, stream, nbr, num_out, max_voxels, K, row_weight, w, bsum);
+    hipLaunchKernelGGL(tile_cuts, dim3(blocks), dim3(kBlock), 0, stream, num_out, max_voxels, gemm_compute_units(), target_rows, row_weight, w,
                        bsum, hdr);
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;

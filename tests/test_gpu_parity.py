@@ -454,10 +454,11 @@ def test_sparse_layers_of_the_backbone(layer):
     cbuf[:n] = coors
     assert np.array_equal(O.canonical_rulebook(pairs, num, cbuf, oc), O.canonical_rulebook(o_pairs, o_num, coors, o_oc))
     o_out = O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv)
-    assert_features_close(out, o_out, RTOL_FP32, layer.name)
+    terms = abs_sum_of(feat, w, o_pairs, o_num, mv)
+    assert_features_close(out, o_out, RTOL_FP32, layer.name, abs_sum=terms)
     a = canonical(oc, on, out)
     b = canonical(o_oc, o_on, o_out)
-    assert_features_close(a[1], b[1], RTOL_FP32, layer.name + " (canonical order)")
+    assert_features_close(a[1], b[1], RTOL_FP32, layer.name + " (canonical order)", abs_sum=canonical(o_oc, o_on, terms)[1])
 
 
 def test_sparse_cap_overflow_and_empty():
