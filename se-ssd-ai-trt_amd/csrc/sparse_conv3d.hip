@@ -160,7 +160,14 @@ sp_number(const int32_t* __restrict__ voxel_num, SpParams P, HashTable t, const 
     // 26 000 active ones, three blocks in four would each add up thousands of counts to find nothing to number).
     int active = (int)(((int64_t)clamp_count(voxel_num, P.max_voxels) * P.Kc + kBlock - 1) / kBlock);
     active = active < n_blocks ? active : n_blocks;
-    if (b > 0 && b >= active) return;
+    if (b >= active) {
+        // (no active input row at all: block 0 still owes the count; the words sp_flags left unwritten are not read)
+        if (b == 0 && threadIdx.x == 0) {
+            *out_num = 0;
+            meta[1] = 0;
+        }
+        return;
+    }
     const int upto = b == 0 ? active : b;  // block 0 computes the total
     uint32_t part = 0;
     for (int j = threadIdx.x; j < upto; j += kBlock) part += block_counts[j];

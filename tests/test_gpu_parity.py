@@ -476,6 +476,16 @@ def test_sparse_cap_overflow_and_empty():
     assert o_st & D.SESSD_STATUS_VOXEL_OVERFLOW and conv.status() & D.SESSD_STATUS_VOXEL_OVERFLOW
     assert on == o_on == mv and np.array_equal(oc, o_oc) and np.array_equal(num, o_num)
     assert_features_close(out, O.gather_gemm_scatter(feat, w, o_pairs, o_num, mv), RTOL_FP32, "capped sparse layer")
+    # an empty frame through the same plugin and workspace, which still hold the full frame's tickets and flags
+    cbuf = np.zeros((mv, 4), np.int32)
+    cbuf[:n] = coors
+    fbuf = np.zeros((mv, layer.cin), np.float32)
+    fbuf[:n] = feat
+    out2, oc2, on2 = conv(dev(fbuf), dev(cbuf), dev(np.array([0], np.int32)))
+    num2 = conv.export_rulebook()[1]
+    torch.cuda.synchronize()
+    assert int(to_np(on2)[0]) == 0 and not to_np(out2).any() and not to_np(oc2).any() and not to_np(num2).any()
+    assert conv.status() == 0
     conv, out, oc, on, pairs, num = run_sparse(layer, coors, 0, feat, w, mv, ig)
     assert on == 0 and np.all(out == 0) and np.all(oc == 0) and np.all(num == 0)
 
