@@ -145,6 +145,9 @@ conv_wide(const float* __restrict__ in, float* __restrict__ out, const void* __r
         s_epi[tid] = epi_scale;
         s_epi[COUT + tid] = epi_shift;
     }
+    // zero this wave's partial tile (while the lists are on their way)
+    float* part = s_part + wave * kTileRows * LDP;
+    for (int t = lane; t < rows * LDP / 4; t += 64) reinterpret_cast<float4*>(part)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int s = 0; s < kListsPerWave; ++s) {
         const int k = wave + s * kWaves;
@@ -163,9 +166,6 @@ conv_wide(const float* __restrict__ in, float* __restrict__ out, const void* __r
         }
         if (lane == 0) s_cnt[k] = base;
     }
-    // zero this wave's partial tile
-    float* part = s_part + wave * kTileRows * LDP;
-    for (int t = lane; t < rows * LDP / 4; t += 64) reinterpret_cast<float4*>(part)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
 
     // offsets of this wave's group: ranked by their number of 16-pair blocks (ballots: lane k holds offset k)
