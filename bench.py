@@ -317,7 +317,7 @@ def measure(config, args, torch, frames=None, points_override=None, deep=True, w
                 "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None}
     # (FP16 3x3x3 layers from 32 channels up run on the tall-tile kernel, FP32 64 -> 64 on the one-tile-per-unit
     # kernel, everything else on the split-K one)
-    kname = ("conv_tall<%d, %d," if half else "conv_wide<%d, %d>" if dom_c == 64 else "conv_mfma<float, %d, %d,") % (dom_c, dom_c)
+    kname = ("conv_tall<%d, %d," if half else "conv_wide<%d, %d," if dom_c == 64 else "conv_mfma<float, %d, %d,") % (dom_c, dom_c)
     traffic, fresh = profiled_traffic(kname, config, dtype)
     roof["traffic"] = traffic
     roof.update({"traffic_source": "profiles/frame_pipeline_config%d_%s.md (rocprofv3 FETCH_SIZE/WRITE_SIZE), collected on %s"

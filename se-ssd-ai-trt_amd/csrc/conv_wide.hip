@@ -44,7 +44,10 @@ __device__ __forceinline__ void mma16(const float4& w, const float4& x, v4f& acc
     acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w.w, x.w, acc, 0, 0, 0);
 }
 
-template <int CIN, int COUT>
+// DENSE: the epilogue also scatters the rows into a dense tensor (the layer in front of sparse2Dense).  A variant of
+// its own because the scatter's addresses cost ten registers, and what this kernel leaves of the register file is
+// what the coordinate kernels of the frame's other branch run in beside it.
+template <int CIN, int COUT, bool DENSE>
 __global__ void __launch_bounds__(kWaves * 64)
 conv_wide(const float* __restrict__ in, float* __restrict__ out, const void* __restrict__ Wp,
           const int32_t* __restrict__ nbr, const int32_t* __restrict__ num_out, int max_voxels, int K,
@@ -304,7 +307,7 @@ conv_wide(const float* __restrict__ in, float* __restrict__ out, const void* __r
             o[e] = s;
         }
         *reinterpret_cast<float4*>(out + (size_t)(row0 + r) * COUT + ec4) = make_float4(o[0], o[1], o[2], o[3]);
-        if (dt.dense) {  // the sparse2Dense scatter of this row, fused (uniform branch)
+        if (DENSE && dt.dense) {  // the sparse2Dense scatter of this row, fused (uniform branch)
             const int4 cc = reinterpret_cast<const int4*>(dt.coors)[row0 + r];  // (b,z,y,x)
             if (cc.x != 0 || cc.y < 0 || cc.y >= dt.D || cc.z < 0 || cc.z >= dt.H || cc.w < 0 || cc.w >= dt.W) {
                 if (dt.status && ec4 == 0) atomicOr(dt.status, SESSD_STATUS_BAD_COORD);
@@ -328,10 +331,16 @@ int launch(const GemmArgs& a, hipStream_t stream) {
         return SESSD_E_UNSUPPORTED;
     const int num_cu = gemm_compute_units();
     const unsigned blocks = (unsigned)num_cu;
-    hipLaunchKernelGGL((conv_wide<CIN, COUT>), dim3(blocks), dim3(kWaves * 64), 0, stream,
-                       static_cast<const float*>(a.in_feat), static_cast<float*>(a.out_feat), a.w_packed, a.nbr,
-                       a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows, num_cu, a.tiles,
-                       a.dense);
+    if (a.dense.dense)
+        hipLaunchKernelGGL((conv_wide<CIN, COUT, true>), dim3(blocks), dim3(kWaves * 64), 0, stream,
+                           static_cast<const float*>(a.in_feat), static_cast<float*>(a.out_feat), a.w_packed, a.nbr,
+                           a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows, num_cu, a.tiles,
+                           a.dense);
+    else
+        hipLaunchKernelGGL((conv_wide<CIN, COUT, false>), dim3(blocks), dim3(kWaves * 64), 0, stream,
+                           static_cast<const float*>(a.in_feat), static_cast<float*>(a.out_feat), a.w_packed, a.nbr,
+                           a.num_out, a.max_voxels, a.K, a.scale, a.shift, a.relu, a.write_pad_rows, num_cu, a.tiles,
+                           a.dense);
     SESSD_HIP_TRY(hipGetLastError());
     return SESSD_OK;
 }

@@ -21,7 +21,7 @@ def test_entry_points_exist():
 def test_bench_reads_the_committed_traffic_figure():
     sys.path.insert(0, ROOT)
     import bench
-    t, fresh = bench.profiled_traffic("conv_wide<64, 64>", 3, "fp32")
+    t, fresh = bench.profiled_traffic("conv_wide<64, 64,", 3, "fp32")
     assert t is not None and 5e6 < t < 1e8                      # bytes per launch, from profiles/
     assert isinstance(fresh, bool)                              # whether profiles/ was collected on this kernel source
     assert bench.profiled_traffic("no_such_kernel", 3, "fp32")[0] is None
