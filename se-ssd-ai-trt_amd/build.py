@@ -27,11 +27,11 @@ def sources():
 
 def headers():
     return (sorted(glob.glob(os.path.join(SRC_DIR, "*.h"))) + [os.path.join(HERE, "..", "include", "sessd3d.h")] +
-            [os.path.join(HERE, "examples", "run_frame.c")])
+            [os.path.join(HERE, "examples", "run_frame.c"), os.path.join(HERE, "examples", "gather_order.hip")])
 
 
 def is_stale():
-    if not os.path.exists(LIB) or not os.path.exists(os.path.join(HERE, "lib", "run_frame")):
+    if not os.path.exists(LIB) or not os.path.exists(os.path.join(HERE, "lib", "run_frame")) or not os.path.exists(GATHER_ORDER):
         return True
     t = os.path.getmtime(LIB)
     return any(os.path.getmtime(p) > t for p in sources() + headers())
@@ -64,6 +64,7 @@ def build(force=True, jobs=8, verbose=False):
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stdout)
     build_example()
+    build_gather_order()
     return LIB
 
 
@@ -83,6 +84,19 @@ def build_example():
     if r.returncode != 0:
         raise RuntimeError("building the C example failed:\n" + r.stdout)
     return EXAMPLE
+
+
+GATHER_ORDER_SRC = os.path.join(HERE, "examples", "gather_order.hip")
+GATHER_ORDER = os.path.join(HERE, "lib", "gather_order")
+
+
+def build_gather_order():
+    """The stand-alone measurement behind the order of conv_wide.hip's row requests (examples/gather_order.hip)."""
+    cmd = [HIPCC] + [f for f in FLAGS if f != "-fPIC"] + [GATHER_ORDER_SRC, "-o", GATHER_ORDER]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building examples/gather_order.hip failed:\n" + r.stdout)
+    return GATHER_ORDER
 
 
 if __name__ == "__main__":
